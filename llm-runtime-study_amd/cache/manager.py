@@ -5,6 +5,7 @@ What each schedule entry of the model keeps between steps is declared by its mix
   PagedKVNeed(nkv, d, window, dtype, value_dim)  keys and values of every position, or of a sliding window, kept in `dtype`
                                (None: the run's activation dtype); value_dim: rows of a value page if not d, 0: key pages alone;
   StateNeed(shape, dtype)      a state of fixed size;
+  BothNeeds(paged, state)      pages and a state (two mixers side by side in one layer);
   ("from", j)                  nothing of its own: it reads the cache of entry j;
   None                         nothing.
 Entries whose paged needs are equal form a group.  A group has a page pool of its own, one
@@ -45,7 +46,7 @@ import numpy as np
 import torch
 
 from ..errors import KVCacheError
-from ..parts import PagedKVNeed, StateNeed
+from ..parts import BothNeeds, PagedKVNeed, StateNeed
 from .pages import PagePool
 
 
@@ -107,6 +108,12 @@ class CacheManager:
         by_need: dict[PagedKVNeed, PagedGroup] = {}
         for position, need in enumerate(needs):
             cache = LayerCache()
+            if isinstance(need, BothNeeds):
+                # the state rows here, the pages below as for a paged need alone
+                self.state_entries.append(position)
+                if allocate_storage:
+                    cache.state = torch.zeros((max_requests + 1, *need.state.shape), dtype=need.state.dtype, device=self.device)
+                need = need.paged
             if isinstance(need, PagedKVNeed):
                 if need not in by_need:
                     by_need[need] = PagedGroup(need, [], num_pages)
@@ -222,7 +229,8 @@ class CacheManager:
         if window is None:
             return blocks
         step = tokens if max_step_tokens is None else max_step_tokens
-        return min(blocks, -(-window // self.page_size) + -(-step // self.page_size) + 2)
+        kept = -(-self.groups[group].need.keep_first // self.page_size)
+        return min(blocks, -(-window // self.page_size) + -(-step // self.page_size) + 2 + kept)
 
     # -------------------------------------------------------------- admission
     def can_admit(self, tokens: int, max_step_tokens: int | None = None) -> bool:
@@ -315,12 +323,14 @@ class CacheManager:
             dead_blocks = max(0, (request.length - window + 1) // self.page_size)
             table = request.tables[index]
             dead_blocks = min(dead_blocks, len(table))
-            pages = [table[b] for b in range(request.first_live[index], dead_blocks) if table[b] >= 0]
-            for b in range(request.first_live[index], dead_blocks):
+            # the pages of the first keep_first positions stay: those keys are seen for good
+            first = max(request.first_live[index], -(-group.need.keep_first // self.page_size))
+            pages = [table[b] for b in range(first, dead_blocks) if table[b] >= 0]
+            for b in range(first, dead_blocks):
                 table[b] = -1
-            if dead_blocks > request.first_live[index]:
-                group.host_table[request.slot, request.first_live[index]:dead_blocks] = -1
-                self._touch(index, request.slot, request.first_live[index], dead_blocks)
+            if dead_blocks > first:
+                group.host_table[request.slot, first:dead_blocks] = -1
+                self._touch(index, request.slot, first, dead_blocks)
                 request.first_live[index] = dead_blocks
             group.pool.free(pages)
             freed += len(pages)

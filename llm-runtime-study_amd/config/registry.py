@@ -72,8 +72,10 @@ def _load_builtin() -> None:
     _builtin_loaded = True
     from ..models.qwen3 import build_spec
     from ..text.chat import format_qwen3_chat
+    from ..models.kaposun import build_spec as build_kaposun
     from ..models.napizen import build_spec as build_napizen
     from ..models.nobodra import build_spec as build_nobodra
+    from .kaposun import KaposunConfig
     from .napizen import NapizenConfig
     from .nobodra import NobodraConfig
     from .qwen3 import Qwen3Config
@@ -84,6 +86,8 @@ def _load_builtin() -> None:
         register_architecture(NobodraConfig.ARCHITECTURE, NobodraConfig, build_nobodra)      # token ids only: it has no chat template
     if NapizenConfig.ARCHITECTURE not in _ARCHITECTURES:
         register_architecture(NapizenConfig.ARCHITECTURE, NapizenConfig, build_napizen)      # token ids only as well
+    if KaposunConfig.ARCHITECTURE not in _ARCHITECTURES:
+        register_architecture(KaposunConfig.ARCHITECTURE, KaposunConfig, build_kaposun)      # token ids only
     import importlib
     import os
 

@@ -22,18 +22,19 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 constexpr float RESCALE_STEP = 8.0f;
 
 // ---------------------------------------------------------- generic kernel
-// One workgroup per (query token, query head); any head_dim up to 4 * threads.
+// One workgroup per (query token, query head); any head_dim, values of any size dv up to 4 * threads.  keep_first: with a
+// window, the keys at positions below keep_first stay visible however far back they lie (they keep their positions).
 template <typename T, int THREADS>
 __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
     T* __restrict__ out, int out_stride, const T* __restrict__ q, int q_stride,
     const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_request,
-    const int* __restrict__ positions, int nq, int nkv, int d, int page_size, float scale,
-    int window) {
+    const int* __restrict__ positions, int nq, int nkv, int d, int dv, int page_size, float scale,
+    int window, int keep_first) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   float* qs = smem;                           // [d]
   float* probs = qs + d + d % 2;              // [THREADS]
-  int64_t* bases = (int64_t*)(probs + THREADS);  // [THREADS] element offset of each key's (page, kv head) block
+  int64_t* bases = (int64_t*)(probs + THREADS);  // [THREADS] index of each key's (page, kv head) block
   int* offsets = (int*)(bases + THREADS);        // [THREADS] slot of each key inside its page
   __shared__ float scratch[16];
 
@@ -42,6 +43,7 @@ __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
   const int pos = positions[token];
   const int kv_head = head / (nq / nkv);
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int kept = lo > 0 ? (keep_first < lo ? keep_first : lo) : 0;    // keys 0 .. kept-1 are seen besides lo .. pos
   const int* table = block_table + (int64_t)request * table_stride;
 
   for (int i = tid; i < d; i += THREADS) qs[i] = to_float(q[(int64_t)token * q_stride + (int64_t)head * d + i]);
@@ -49,16 +51,21 @@ __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
 
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
   float running_max = -INFINITY, running_sum = 0.f;
-  for (int tile = (lo / THREADS) * THREADS; tile <= pos; tile += THREADS) {
+  const int lo_tile = (lo / THREADS) * THREADS;
+  for (int tile = kept > 0 ? 0 : lo_tile; tile <= pos; tile += THREADS) {
+    if (tile >= kept && tile < lo_tile) {     // nothing to see between the kept keys and the window
+      tile = lo_tile - THREADS;
+      continue;
+    }
     const int key = tile + tid;
-    const bool valid = key >= lo && key <= pos;
+    const bool valid = key <= pos && (key >= lo || key < kept);
     float score = -INFINITY;
     int64_t base = 0;
     const int off = key % page_size;
     if (valid) {
       const int64_t page = table[key / page_size];
-      base = (page * nkv + kv_head) * page_size * d;
-      const T* kr = k_pages + base + (int64_t)off * d;
+      base = page * nkv + kv_head;
+      const T* kr = k_pages + (base * page_size + off) * d;
       float dot = 0.f;
       if (sizeof(T) == 4 && d % 4 == 0 && ((uintptr_t)k_pages % 16) == 0) {
         // float32 rows, 16 bytes a load; the products are added up in the same order as one by one
@@ -82,27 +89,20 @@ __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
     running_sum = running_sum * alpha + tile_sum;
     running_max = new_max;
     probs[tid] = p;
-    bases[tid] = base;
+    bases[tid] = base * page_size * dv;
     offsets[tid] = off;
     __syncthreads();
     const int count = (pos - tile + 1 < THREADS) ? pos - tile + 1 : THREADS;
+    const bool whole = tile >= lo;             // every key of the tile up to pos is seen, so each has a page to read from
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       const int dim = tid + c * THREADS;
-      if (dim < d) {
+      if (dim < dv) {
         float a = acc[c] * alpha;
-        if (sizeof(T) == 4 && page_size % 4 == 0 && THREADS % 4 == 0 && ((uintptr_t)v_pages % 16) == 0) {
+        int j = 0;
+        if (whole && sizeof(T) == 4 && page_size % 4 == 0 && THREADS % 4 == 0 && ((uintptr_t)v_pages % 16) == 0) {
           // four keys that lie side by side in a (transposed) page in one load of 16 bytes; added in key order as below
-          int j = 0;
           for (; j + 4 <= count; j += 4) {
-            if (tile + j < lo) {                                 // keys before the window have no page to read from
-#pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                const float pj = probs[j + e];
-                if (pj != 0.f) a = fmaf(pj, to_float(v_pages[bases[j + e] + (int64_t)dim * page_size + offsets[j + e]]), a);
-              }
-              continue;
-            }
             const floatx4 vv = *(const floatx4*)((const float*)v_pages + bases[j] + (int64_t)dim * page_size + offsets[j]);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -110,15 +110,10 @@ __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
               if (pj != 0.f) a = fmaf(pj, vv[e], a);
             }
           }
-          for (; j < count; ++j) {
-            const float pj = probs[j];
-            if (pj != 0.f) a = fmaf(pj, to_float(v_pages[bases[j] + (int64_t)dim * page_size + offsets[j]]), a);
-          }
-        } else {
-          for (int j = 0; j < count; ++j) {
-            const float pj = probs[j];
-            if (pj != 0.f) a = fmaf(pj, to_float(v_pages[bases[j] + (int64_t)dim * page_size + offsets[j]]), a);
-          }
+        }
+        for (; j < count; ++j) {
+          const float pj = probs[j];
+          if (pj != 0.f) a = fmaf(pj, to_float(v_pages[bases[j] + (int64_t)dim * page_size + offsets[j]]), a);
         }
         acc[c] = a;
       }
@@ -129,7 +124,7 @@ __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
     const int dim = tid + c * THREADS;
-    if (dim < d) out[(int64_t)token * out_stride + (int64_t)head * d + dim] = from_float<T>(acc[c] * inv);
+    if (dim < dv) out[(int64_t)token * out_stride + (int64_t)head * dv + dim] = from_float<T>(acc[c] * inv);
   }
 }
 
@@ -1520,12 +1515,13 @@ LRS_API int lrs_compute_units() { return compute_units(); }
 LRS_API int lrs_attention(void* out, int out_stride, const void* q, int q_stride, const void* k_pages,
                           const void* v_pages, const int* block_table, int table_stride,
                           const int* token_request, const int* positions, int dtype, int tokens,
-                          int nq, int nkv, int d, int page_size, float scale, int window,
+                          int nq, int nkv, int d, int dv, int page_size, float scale, int window, int keep_first,
                           void* stream) {
-  LRS_REQUIRE(tokens > 0 && nq > 0 && nkv > 0 && d > 0 && page_size > 0, "attention: bad sizes tokens=%d nq=%d nkv=%d d=%d page=%d", tokens, nq, nkv, d, page_size);
+  // value pages [P, nkv, dv, page]; out rows hold nq heads of dv values
+  LRS_REQUIRE(tokens > 0 && nq > 0 && nkv > 0 && d > 0 && dv > 0 && page_size > 0, "attention: bad sizes tokens=%d nq=%d nkv=%d d=%d dv=%d page=%d", tokens, nq, nkv, d, dv, page_size);
   LRS_REQUIRE(nq % nkv == 0, "attention: %d query heads do not divide into %d kv heads", nq, nkv);
-  LRS_REQUIRE(d <= 512, "attention: head_dim %d above the supported 512", d);
-  LRS_REQUIRE(window >= 0, "attention: window must be >= 0 (0 = none)");
+  LRS_REQUIRE(d <= 512 && dv <= 512, "attention: head sizes %d and %d above the supported 512", d, dv);
+  LRS_REQUIRE(window >= 0 && keep_first >= 0, "attention: window and keep_first must be >= 0 (0 = none)");
   constexpr int THREADS = 128;
   dim3 grid(tokens, nq);
   const size_t lds = sizeof(float) * (d + d % 2 + THREADS) + (sizeof(int64_t) + sizeof(int)) * THREADS + 16;
@@ -1533,11 +1529,11 @@ LRS_API int lrs_attention(void* out, int out_stride, const void* q, int q_stride
   if (dtype == LRS_F32)
     attention_generic_kernel<float, THREADS><<<grid, THREADS, lds, s>>>(
         (float*)out, out_stride, (const float*)q, q_stride, (const float*)k_pages, (const float*)v_pages,
-        block_table, table_stride, token_request, positions, nq, nkv, d, page_size, scale, window);
+        block_table, table_stride, token_request, positions, nq, nkv, d, dv, page_size, scale, window, keep_first);
   else if (dtype == LRS_BF16)
     attention_generic_kernel<bf16, THREADS><<<grid, THREADS, lds, s>>>(
         (bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)v_pages,
-        block_table, table_stride, token_request, positions, nq, nkv, d, page_size, scale, window);
+        block_table, table_stride, token_request, positions, nq, nkv, d, dv, page_size, scale, window, keep_first);
   else
     return lrs_fail("attention: unknown dtype %d", dtype);
   return lrs_check_launch("attention");

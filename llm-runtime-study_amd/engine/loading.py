@@ -66,11 +66,14 @@ RESERVE_MARGIN = 3 << 29          # the step's buffers (activations, logits, met
 def engine_bytes(model: DecoderModel, dtype: torch.dtype, page_size: int, num_pages: int) -> int:
     """About how many bytes of device memory an engine of `model` (bound or not) holds: its weights in `dtype`
     and its cache pool of `num_pages` pages; an estimate (integer tables and 32-bit norms count as `dtype`)."""
-    from ..parts import PagedKVNeed, StateNeed
+    from ..parts import BothNeeds, PagedKVNeed, StateNeed
 
     item = torch.empty(0, dtype=dtype).element_size()
-    total = sum(math.prod(spec.shape) for spec in model.tensors().values()) * item
+    total = sum(math.prod(abs(size) for size in spec.shape) for spec in model.tensors().values()) * item
+    needs = []
     for need in model.cache_needs():
+        needs.extend((need.paged, need.state) if isinstance(need, BothNeeds) else (need,))
+    for need in needs:
         if isinstance(need, PagedKVNeed):
             size = item if need.dtype is None else torch.empty(0, dtype=need.dtype).element_size()
             total += 2 * need.num_kv_heads * need.head_dim * size * page_size * (num_pages + 1)

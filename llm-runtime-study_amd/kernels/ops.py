@@ -124,7 +124,18 @@ _SIGNATURES = {
                                             c_void_p, c_int64, c_void_p]),
     "lrs_norm_begin_parts": (c_int, [c_int]),
     "lrs_attention": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
-                              c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
+                              c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p]),
+    "lrs_qkv_norm_prep": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
+                                  c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    "lrs_sigmoid_gate": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    "lrs_axpby": (c_int, [c_void_p, c_void_p, c_float, c_void_p, c_float, c_int, c_int, c_void_p, c_float, c_void_p, c_int, c_void_p]),
+    "lrs_activation": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int, c_void_p]),
+    "lrs_delta_rule_channels": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
+                                        c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
+                                        c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p]),
+    "lrs_ssm": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
+                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_float,
+                        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "lrs_attention_decode": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                      c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int,
                                      c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_void_p]),
@@ -205,11 +216,11 @@ def library():
 #
 # PLAN_OPS fixes the number of each entry point inside a plan; csrc/plan_dispatch.inc, made from this list
 # and _SIGNATURES by kernels/plan_codegen.py, is the other side (a test keeps the two in step).
-PLAN_OPS = ("lrs_add_into", "lrs_add_rmsnorm", "lrs_advance_decode", "lrs_advance_slots", "lrs_attention", "lrs_attention_decode",
-            "lrs_attention_prefill", "lrs_choose_tokens", "lrs_choose_tokens_split", "lrs_copy_to_pinned", "lrs_delta_rule", "lrs_embed", "lrs_fill_i32",
+PLAN_OPS = ("lrs_activation", "lrs_add_into", "lrs_add_rmsnorm", "lrs_advance_decode", "lrs_advance_slots", "lrs_attention", "lrs_attention_decode",
+            "lrs_attention_prefill", "lrs_axpby", "lrs_choose_tokens", "lrs_choose_tokens_split", "lrs_copy_to_pinned", "lrs_delta_rule", "lrs_delta_rule_channels", "lrs_embed", "lrs_fill_i32",
             "lrs_filter_logits", "lrs_gather_rows", "lrs_gemm", "lrs_gemm_lines_add_rmsnorm", "lrs_gemm_mid_add_norm_begin", "lrs_gemm_mid_qk_prep", "lrs_gemm_mid_scaled",
             "lrs_gemm_norm_chain", "lrs_head_gemm", "lrs_latent_attention", "lrs_latent_attention_groups", "lrs_latent_prep", "lrs_layernorm", "lrs_library_gemm", "lrs_moe_align", "lrs_moe_combine", "lrs_moe_experts", "lrs_moe_route", "lrs_moe_route_align", "lrs_norm_add",
-            "lrs_qk_prep", "lrs_rmsnorm", "lrs_rope_table", "lrs_round_rows", "lrs_scale_add_layernorm", "lrs_scale_rows", "lrs_silu_mul", "lrs_soft_cap")
+            "lrs_qk_prep", "lrs_qkv_norm_prep", "lrs_rmsnorm", "lrs_rope_table", "lrs_round_rows", "lrs_scale_add_layernorm", "lrs_scale_rows", "lrs_sigmoid_gate", "lrs_silu_mul", "lrs_soft_cap", "lrs_ssm")
 _PLAN_INDEX = {name: index for index, name in enumerate(PLAN_OPS)}
 
 
@@ -950,14 +961,15 @@ def scale_rows(out: torch.Tensor, x: torch.Tensor, sumsq: torch.Tensor, eps: flo
 
 # -------------------------------------------------------------- attention
 def attention(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
-              token_request: torch.Tensor, positions: torch.Tensor, nq: int, scale: float, window: int = 0) -> None:
-    """out [T, nq*d]; q [T, >= nq*d] (leading nq*d columns of each row); key pages [P, nkv, page, d],
-    value pages [P, nkv, d, page]."""
+              token_request: torch.Tensor, positions: torch.Tensor, nq: int, scale: float, window: int = 0, keep_first: int = 0) -> None:
+    """out [T, nq*dv]; q [T, >= nq*d] (leading nq*d columns of each row); key pages [P, nkv, page, d],
+    value pages [P, nkv, dv, page].  window: a token at p sees keys above p - window; keep_first: and those below keep_first."""
     tokens = out.shape[0]
-    _need(k_pages.dim() == 4 and k_pages.is_contiguous() and v_pages.is_contiguous(), "attention: pages must be contiguous")
+    _need(k_pages.dim() == 4 and v_pages.dim() == 4 and k_pages.is_contiguous() and v_pages.is_contiguous(), "attention: pages must be contiguous")
     _, nkv, page_size, d = k_pages.shape
-    _need(v_pages.shape == (k_pages.shape[0], nkv, d, page_size), "attention: key pages must be [P, nkv, page, d] and value pages [P, nkv, d, page]")
-    _need(out.shape[1] == nq * d and q.shape[0] == tokens and q.shape[1] >= nq * d, "attention: q/out widths do not match nq*d")
+    dv = v_pages.shape[2]
+    _need(v_pages.shape == (k_pages.shape[0], nkv, dv, page_size), "attention: key pages must be [P, nkv, page, d] and value pages [P, nkv, dv, page]")
+    _need(out.shape[1] == nq * dv and q.shape[0] == tokens and q.shape[1] >= nq * d, "attention: q/out widths do not match nq*d and nq*dv")
     _need(q.dtype == k_pages.dtype == v_pages.dtype == out.dtype, "attention: q, pages and out must share a dtype")
     _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.stride(1) == 1, "attention: block_table must be int32 [R, blocks]")
     for name, t in (("token_request", token_request), ("positions", positions)):
@@ -965,7 +977,66 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages
     _launch("lrs_attention", 
         _dev(out, "out"), _rows(out, "out"), _dev(q, "q"), _rows(q, "q"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"),
         _dev(block_table, "block_table"), block_table.stride(0), _dev(token_request, "token_request"), _dev(positions, "positions"),
-        dtype_code(q.dtype), tokens, nq, nkv, d, page_size, scale, window, _stream())
+        dtype_code(q.dtype), tokens, nq, nkv, d, dv, page_size, scale, window, keep_first, _stream())
+
+
+def qkv_norm_prep(qkv: torch.Tensor, nq: int, nkv: int, d: int, dv: int, q_weight, k_weight, eps: float, cos, sin,
+                  k_pages: torch.Tensor, v_pages: torch.Tensor, slots: torch.Tensor, page_size: int) -> None:
+    """The rows of `qkv` [T, >= nq*d + nkv*d + nkv*dv] (q | k | v | whatever follows): q and k each divided by the root mean
+    square of the whole part (all heads at once) and multiplied by a weight per column (float32 [nq*d], [nkv*d]; None: no
+    norm), the first 2 * cos.shape[1] dims of every head rotated; q in place, k and v into the pages."""
+    tokens = qkv.shape[0]
+    stride = _rows(qkv, "qkv")
+    _need(qkv.shape[1] >= (nq + nkv) * d + nkv * dv, "qkv_norm_prep: the rows hold fewer than q, k and v")
+    rot_half = 0
+    if cos is not None:
+        rot_half = cos.shape[1]
+        _need(cos.shape[0] >= tokens and sin.shape == cos.shape and cos.is_contiguous() and sin.is_contiguous()
+              and cos.dtype == torch.float32 and sin.dtype == torch.float32, "qkv_norm_prep: rotary tables must be float32 [T, half]")
+    if q_weight is not None:
+        _need(k_weight is not None and q_weight.numel() == nq * d and k_weight.numel() == nkv * d and q_weight.dtype == k_weight.dtype == torch.float32
+              and q_weight.is_contiguous() and k_weight.is_contiguous(), "qkv_norm_prep: norm weights must be float32 [nq*d] and [nkv*d]")
+    _need(k_pages.dim() == 4 and k_pages.shape[1:] == (nkv, page_size, d) and v_pages.shape == (k_pages.shape[0], nkv, dv, page_size),
+          f"qkv_norm_prep: key pages must be [pages, {nkv}, {page_size}, {d}] and value pages [pages, {nkv}, {dv}, {page_size}]")
+    _need(k_pages.is_contiguous() and v_pages.is_contiguous() and k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype,
+          "qkv_norm_prep: pages must be contiguous and of the activation dtype")
+    _need(slots.dtype == torch.int32 and slots.numel() >= tokens and slots.is_contiguous(), "qkv_norm_prep: slots must be int32 [T]")
+    _launch("lrs_qkv_norm_prep", _dev(qkv, "qkv"), dtype_code(qkv.dtype), tokens, stride, nq, nkv, d, dv,
+            None if q_weight is None else _dev(q_weight, "q_weight"), None if k_weight is None else _dev(k_weight, "k_weight"), eps,
+            None if cos is None else cos.data_ptr(), None if sin is None else sin.data_ptr(), rot_half, _dev(k_pages, "k_pages"),
+            _dev(v_pages, "v_pages"), _dev(slots, "slots"), page_size, _stream())
+
+
+def sigmoid_gate(out: torch.Tensor, gate: torch.Tensor) -> None:
+    """out *= sigmoid(gate), both [T, C] with rows that may be strided (a gate that lies in a wider projection row)."""
+    _need(out.shape == gate.shape and out.dtype == gate.dtype and out.dim() == 2, "sigmoid_gate: out and gate must be [T, C] of one dtype")
+    _launch("lrs_sigmoid_gate", _dev(out, "out"), _rows(out, "out"), _dev(gate, "gate"), _rows(gate, "gate"), dtype_code(out.dtype),
+            out.shape[0], out.shape[1], _stream())
+
+
+def axpby(out: torch.Tensor, a: torch.Tensor, alpha: float, b: torch.Tensor, beta: float, norm_weight: torch.Tensor | None = None,
+          eps: float = 0.0, normed: torch.Tensor | None = None) -> None:
+    """out = alpha * a + beta * b over contiguous float32 [T, C] (out may be a or b).  norm_weight (float32 [C]): `normed`
+    [T, C] also receives the RMS norm of the new rows times the weight."""
+    for name, t in (("out", out), ("a", a), ("b", b)):
+        _need(t.dtype == torch.float32 and t.is_contiguous() and t.shape == out.shape and t.dim() == 2, f"axpby: {name} must be contiguous float32 [T, C]")
+    if norm_weight is not None:
+        _need(norm_weight.dtype == torch.float32 and norm_weight.numel() == out.shape[1] and norm_weight.is_contiguous(), "axpby: the norm's weight must be float32 [C]")
+        _need(normed is not None and normed.shape == out.shape and normed.is_contiguous(), "axpby: the normalised rows need a contiguous [T, C] buffer")
+    _launch("lrs_axpby", _dev(out, "out"), _dev(a, "a"), alpha, _dev(b, "b"), beta, out.shape[0], out.shape[1],
+            None if norm_weight is None else _dev(norm_weight, "norm_weight"), eps, None if norm_weight is None else _dev(normed, "normed"),
+            0 if norm_weight is None else dtype_code(normed.dtype), _stream())
+
+
+ACTIVATIONS = {"gelu": 0, "gelu_tanh": 1, "silu": 2, "relu": 3}
+
+
+def activation(out: torch.Tensor, x: torch.Tensor, kind: str) -> None:
+    """out = act(x) elementwise (out may be x): "gelu" (0.5 x (1 + erf(x / sqrt 2))), "gelu_tanh", "silu", "relu"."""
+    _need(kind in ACTIVATIONS, f"activation: unknown kind {kind!r}; known: {', '.join(ACTIVATIONS)}")
+    _need(out.shape == x.shape and out.dtype == x.dtype and out.is_contiguous() and x.is_contiguous() and x.numel() > 0,
+          "activation: out and x must be contiguous, of one shape and dtype")
+    _launch("lrs_activation", _dev(out, "out"), _dev(x, "x"), dtype_code(x.dtype), x.numel(), ACTIVATIONS[kind], _stream())
 
 
 DECODE_HEAD_DIMS = (32, 64, 96, 128, 192)
@@ -1215,6 +1286,74 @@ def delta_rule(out: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, token
             requests, _dev(token_request, "token_request"), _dev(cu_seqlens, "cu_seqlens"), _dev(slot_ids, "slot_ids"), _dev(state, "state"),
             state.stride(0), _dev(conv_weight, "conv_weight"), taps, kv_heads, heads, dim, vdim, _dev(a_log, "a_log"), _dev(dt_bias, "dt_bias"),
             _dev(norm_weight, "norm_weight"), eps, _dev(qkv, "qkv"), _dev(gates, "gates"), _dev(raw, "raw"), _stream())
+
+
+def delta_rule_channels(out: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, token_request: torch.Tensor, cu_seqlens: torch.Tensor,
+                        slot_ids: torch.Tensor, requests: int, conv_weight: torch.Tensor, kv_heads: int, heads: int, dim: int, vdim: int,
+                        a_log: torch.Tensor, dt_bias: torch.Tensor, norm_weight: torch.Tensor, eps: float, qkv: torch.Tensor, gates: torch.Tensor,
+                        raw: torch.Tensor, decay_up: torch.Tensor, decays: torch.Tensor, gate_up: torch.Tensor) -> None:
+    """The gated delta rule with a decay per head and key channel and a sigmoid output gate, both from inputs of low rank.
+    proj [T, >= C] columns: q (kv_heads*dim) | k (kv_heads*dim) | v (heads*vdim) | step size (heads) | decay input (rank_a) |
+    gate input (rank_g); decay_up float32 [rank_a, heads*dim], dt_bias [heads*dim], gate_up float32 [rank_g, heads*vdim];
+    decays [T, heads*dim] float32 scratch.  Everything else as delta_rule()."""
+    tokens = out.shape[0]
+    channels = 2 * kv_heads * dim + heads * vdim
+    taps = conv_weight.shape[1]
+    rank_a, rank_g = decay_up.shape[0], gate_up.shape[0]
+    _need(out.is_contiguous() and out.shape[1] == heads * vdim, "delta_rule_channels: out must be contiguous [T, heads*vdim]")
+    _need(proj.shape[0] >= tokens and proj.shape[1] >= channels + heads + rank_a + rank_g, "delta_rule_channels: proj holds too few columns")
+    _need(state.dim() == 2 and state.dtype == torch.float32 and state.is_contiguous()
+          and state.shape[1] >= delta_state_floats(heads, kv_heads, dim, vdim, taps), "delta_rule_channels: state rows are too short")
+    _need(conv_weight.shape == (channels, taps) and conv_weight.dtype == torch.float32 and conv_weight.is_contiguous(),
+          f"delta_rule_channels: the convolution's weights must be float32 [{channels}, taps]")
+    for name, t, shape in (("a_log", a_log, (heads,)), ("dt_bias", dt_bias, (heads * dim,)), ("norm_weight", norm_weight, (vdim,)),
+                           ("decay_up", decay_up, (rank_a, heads * dim)), ("gate_up", gate_up, (rank_g, heads * vdim))):
+        _need(t.dtype == torch.float32 and tuple(t.shape) == shape and t.is_contiguous(), f"delta_rule_channels: {name} must be float32 {shape}")
+    for name, t, count in (("token_request", token_request, tokens), ("cu_seqlens", cu_seqlens, requests + 1), ("slot_ids", slot_ids, requests)):
+        _need(t.dtype == torch.int32 and t.numel() >= count and t.is_contiguous(), f"delta_rule_channels: {name} must be int32 [{count}]")
+    for name, t, count in (("qkv", qkv, tokens * channels), ("gates", gates, tokens * 2 * heads), ("raw", raw, tokens * heads * vdim),
+                           ("decays", decays, tokens * heads * dim)):
+        _need(t.dtype == torch.float32 and t.is_contiguous() and t.numel() >= count, f"delta_rule_channels: {name} scratch too small")
+    _launch("lrs_delta_rule_channels", _dev(out, "out"), dtype_code(out.dtype), _dev(proj, "proj"), dtype_code(proj.dtype), _rows(proj, "proj"), tokens,
+            requests, _dev(token_request, "token_request"), _dev(cu_seqlens, "cu_seqlens"), _dev(slot_ids, "slot_ids"), _dev(state, "state"),
+            state.stride(0), _dev(conv_weight, "conv_weight"), taps, kv_heads, heads, dim, vdim, _dev(a_log, "a_log"), _dev(dt_bias, "dt_bias"),
+            _dev(norm_weight, "norm_weight"), eps, _dev(qkv, "qkv"), _dev(gates, "gates"), _dev(raw, "raw"), rank_a, _dev(decay_up, "decay_up"),
+            _dev(decays, "decays"), rank_g, _dev(gate_up, "gate_up"), _stream())
+
+
+def state_space(out: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, token_request: torch.Tensor, cu_seqlens: torch.Tensor,
+                slot_ids: torch.Tensor, requests: int, conv_weight: torch.Tensor, conv_bias: torch.Tensor | None, groups: int, heads: int,
+                state_size: int, vdim: int, a_log: torch.Tensor, dt_bias: torch.Tensor, skip: torch.Tensor, norm_weight: torch.Tensor,
+                norm_parts: int, eps: float, qkv: torch.Tensor, gates: torch.Tensor, raw: torch.Tensor, skipped: torch.Tensor) -> None:
+    """One step of the selective state space recurrence for a ragged batch: per head S <- exp(-exp(a_log) dt) S + dt B x^T,
+    y = S^T C + skip x, then y * silu(z) normalised in `norm_parts` equal parts.  proj [T, >= C] columns: z (heads*vdim) |
+    x (heads*vdim) | B (groups*state_size) | C (groups*state_size) | dt (heads); conv_weight float32 [heads*vdim + 2*groups*state_size,
+    taps] over x | B | C; state [slots, floats] as the delta rule's with dim = state_size; out [T, heads*vdim]."""
+    tokens = out.shape[0]
+    inner = heads * vdim
+    channels = inner + 2 * groups * state_size
+    taps = conv_weight.shape[1]
+    _need(out.is_contiguous() and out.shape[1] == inner, "state_space: out must be contiguous [T, heads*vdim]")
+    _need(proj.shape[0] >= tokens and proj.shape[1] >= inner + channels + heads, "state_space: proj holds too few columns")
+    _need(state.dim() == 2 and state.dtype == torch.float32 and state.is_contiguous()
+          and state.shape[1] >= delta_state_floats(heads, groups, state_size, vdim, taps), "state_space: state rows are too short")
+    _need(conv_weight.shape == (channels, taps) and conv_weight.dtype == torch.float32 and conv_weight.is_contiguous(),
+          f"state_space: the convolution's weights must be float32 [{channels}, taps]")
+    vectors = [("a_log", a_log, heads), ("dt_bias", dt_bias, heads), ("skip", skip, heads), ("norm_weight", norm_weight, inner)]
+    if conv_bias is not None:
+        vectors.append(("conv_bias", conv_bias, channels))
+    for name, t, count in vectors:
+        _need(t.dtype == torch.float32 and t.numel() == count and t.is_contiguous(), f"state_space: {name} must hold {count} float32 values")
+    for name, t, count in (("token_request", token_request, tokens), ("cu_seqlens", cu_seqlens, requests + 1), ("slot_ids", slot_ids, requests)):
+        _need(t.dtype == torch.int32 and t.numel() >= count and t.is_contiguous(), f"state_space: {name} must be int32 [{count}]")
+    for name, t, count in (("qkv", qkv, tokens * channels), ("gates", gates, tokens * 2 * heads), ("raw", raw, tokens * inner), ("skipped", skipped, tokens * inner)):
+        _need(t.dtype == torch.float32 and t.is_contiguous() and t.numel() >= count, f"state_space: {name} scratch too small")
+    _need(norm_parts > 0 and inner % norm_parts == 0, f"state_space: {inner} values do not divide into {norm_parts} parts")
+    _launch("lrs_ssm", _dev(out, "out"), dtype_code(out.dtype), _dev(proj, "proj"), dtype_code(proj.dtype), _rows(proj, "proj"), tokens,
+            requests, _dev(token_request, "token_request"), _dev(cu_seqlens, "cu_seqlens"), _dev(slot_ids, "slot_ids"), _dev(state, "state"),
+            state.stride(0), _dev(conv_weight, "conv_weight"), None if conv_bias is None else _dev(conv_bias, "conv_bias"), taps, groups, heads,
+            state_size, vdim, _dev(a_log, "a_log"), _dev(dt_bias, "dt_bias"), _dev(skip, "skip"), _dev(norm_weight, "norm_weight"), norm_parts,
+            eps, _dev(qkv, "qkv"), _dev(gates, "gates"), _dev(raw, "raw"), _dev(skipped, "skipped"), _stream())
 
 
 # ------------------------------------------------------------------- routed experts

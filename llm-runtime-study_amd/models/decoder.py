@@ -123,7 +123,14 @@ class DecoderModel:
             layer = self.layers[entry.layer]
             kind = getattr(layer, "handover_kind", None)
             if kind is not None:
-                handed = layer.forward(ctx, h, ctx.layer_cache(position), given=handed if handed_kind == kind else None)
+                given = handed if handed_kind == kind else None
+                if getattr(layer, "takes_next_norm", False):
+                    # a block that can leave the next block's norm of the updated stream behind is told which norm that is
+                    following = self.layers[schedule[position + 1].layer] if position + 1 < len(schedule) else None
+                    next_norm = following.first_norm if getattr(following, "handover_kind", None) == kind else None
+                    handed = layer.forward(ctx, h, ctx.layer_cache(position), given=given, next_norm=next_norm)
+                else:
+                    handed = layer.forward(ctx, h, ctx.layer_cache(position), given=given)
                 handed_kind, begun = kind, None
                 continue
             handed = handed_kind = None

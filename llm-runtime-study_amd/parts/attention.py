@@ -14,6 +14,13 @@ value projection: a position's value is its key as projected, before the per-hea
 key matrix is stacked a second time where the value matrix would be, so that every kernel after the product sees
 the usual row of q, k and v heads (the product makes those columns twice, from the same weights and inputs).
 `forward(..., accumulate=False)` stores the output projection into the float32 rows it is given instead of adding to them.
+
+Further forms, each a parameter: `norm_over="projection"` normalises q and k over the whole projection (all heads of a token
+at once, a weight per column) instead of per head; `value_dim` gives the values a size of their own; `keep_first` keeps the
+first positions of a sequence visible behind a window (token i sees j <= i with i - j < window or j < keep_first; the kept
+keys keep their positions); `output_gate` multiplies the heads' outputs by sigmoid(W_g x) before the output projection (the
+gate's matrix is stacked behind q, k and v).  A layer with any of them prepares its heads with `qkv_norm_prep`; its attention
+runs on the matrix cores where the shape allows (values as wide as keys, no kept positions) and in the any-shape kernel otherwise.
 """
 
 from __future__ import annotations
@@ -38,7 +45,8 @@ class GQAAttention(Part):
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, *,
                  position: PartSpec = PartSpec("none"), qk_norm: bool = False, qk_norm_eps: float = 1e-6,
                  bias: bool = False, scale: float | None = None, window: int | None = None,
-                 kv_shared: bool = False, values_from_keys: bool = False):
+                 kv_shared: bool = False, values_from_keys: bool = False, norm_over: str = "head", value_dim: int | None = None,
+                 keep_first: int = 0, output_gate: bool = False):
         for name, value in (("hidden_size", hidden_size), ("num_heads", num_heads), ("num_kv_heads", num_kv_heads), ("head_dim", head_dim)):
             if value <= 0:
                 raise ValueError(f"{name} must be positive, got {value}")
@@ -57,31 +65,50 @@ class GQAAttention(Part):
         if values_from_keys and kv_shared:
             raise ValueError("a layer that owns no keys has no values to take from them")
         self.window, self.kv_shared, self.values_from_keys = window, kv_shared, values_from_keys
+        if norm_over not in ("head", "projection"):
+            raise ValueError(f"norm_over must be 'head' or 'projection', got {norm_over!r}")
+        if value_dim is not None and value_dim <= 0:
+            raise ValueError(f"value_dim must be positive when given, got {value_dim}")
+        if keep_first < 0 or (keep_first and window is None):
+            raise ValueError(f"keep_first must not be negative and needs a window, got {keep_first}")
+        self.norm_over, self.value_dim, self.keep_first, self.output_gate = norm_over, value_dim or head_dim, keep_first, output_gate
+        # the forms that the kernel preparing whole rows serves (see the module's text)
+        self.whole_rows = (qk_norm and norm_over == "projection") or self.value_dim != head_dim or keep_first > 0 or output_gate
+        if self.whole_rows and (kv_shared or values_from_keys or bias or (qk_norm and norm_over == "head")):
+            raise ValueError("a norm over the projection, values of their own size, kept first positions and an output gate come "
+                             "without biases, shared or key-made values and per-head norms")
         self.w_qkv = self.b_qkv = self.w_o = self.q_norm = self.k_norm = None
 
     # ------------------------------------------------------------------ weights
     def tensors(self):
         h, d = self.hidden_size, self.head_dim
         names = ("q_proj",) if self.kv_shared else ("q_proj", "k_proj") if self.values_from_keys else ("q_proj", "k_proj", "v_proj")
-        widths = {"q_proj": self.num_heads * d, "k_proj": self.num_kv_heads * d, "v_proj": self.num_kv_heads * d}
+        widths = {"q_proj": self.num_heads * d, "k_proj": self.num_kv_heads * d, "v_proj": self.num_kv_heads * self.value_dim}
         specs = {f"{n}.weight": TensorSpec((widths[n], h)) for n in names}
         if self.bias:
             specs.update({f"{n}.bias": TensorSpec((widths[n],), role="bias") for n in names})
-        specs["o_proj.weight"] = TensorSpec((h, self.num_heads * d))
+        if self.output_gate:
+            specs["g_proj.weight"] = TensorSpec((self.num_heads * self.value_dim, h))
+        specs["o_proj.weight"] = TensorSpec((h, self.num_heads * self.value_dim))
         if self.qk_norm:
-            specs["q_norm.weight"] = TensorSpec((d,), role="norm")
+            over = d if self.norm_over == "head" else None
+            specs["q_norm.weight"] = TensorSpec((over or widths["q_proj"],), role="norm")
             if not self.kv_shared:
-                specs["k_norm.weight"] = TensorSpec((d,), role="norm")
+                specs["k_norm.weight"] = TensorSpec((over or widths["k_proj"],), role="norm")
         return specs
 
     def bind(self, weights, dtype):
         names = ("q_proj",) if self.kv_shared else ("q_proj", "k_proj", "k_proj") if self.values_from_keys else ("q_proj", "k_proj", "v_proj")
+        if self.output_gate:
+            names += ("g_proj",)
         self.w_qkv = torch.cat([weights[f"{n}.weight"] for n in names], 0).to(dtype).contiguous()
         self.b_qkv = torch.cat([weights[f"{n}.bias"] for n in names], 0).to(dtype).contiguous() if self.bias else None
         self.w_o = weights["o_proj.weight"].to(dtype).contiguous()
         if self.qk_norm:
             self.q_norm = weights["q_norm.weight"]
             self.k_norm = weights["k_norm.weight"] if not self.kv_shared else self.q_norm
+            if self.whole_rows:
+                self.q_norm, self.k_norm = self.q_norm.float().contiguous(), self.k_norm.float().contiguous()
 
     def weight_bytes(self):
         return (self.w_qkv.numel() + self.w_o.numel()) * self.w_o.element_size()
@@ -90,11 +117,14 @@ class GQAAttention(Part):
         if self.window is not None:
             pairs = min(pairs, tokens * self.window)
         # the projections, then scores and weighted values: two products of head_dim per pair and query head
-        return super().flops(tokens, pairs) + 4.0 * pairs * self.num_heads * self.head_dim
+        return super().flops(tokens, pairs) + 2.0 * pairs * self.num_heads * (self.head_dim + self.value_dim)
 
     def cache_need(self):
         if self.kv_shared:
             return None
+        if self.value_dim != self.head_dim or self.keep_first:
+            return PagedKVNeed(self.num_kv_heads, self.head_dim, self.window, value_dim=None if self.value_dim == self.head_dim else self.value_dim,
+                               keep_first=self.keep_first)
         return PagedKVNeed(self.num_kv_heads, self.head_dim, self.window)
 
     @staticmethod
@@ -163,9 +193,11 @@ class GQAAttention(Part):
         t, d, nq = rows_of(x), self.head_dim, self.num_heads
         nkv = 0 if self.kv_shared else self.num_kv_heads
         group = ctx.group(cache.group)
-        qkv = ctx.scratch("attn_qkv", (t, (nq + 2 * nkv) * d), ctx.dtype)
         tables = self.position.tables(ctx)
         cos, sin = tables if tables is not None else (None, None)
+        if self.whole_rows:
+            return self._forward_whole_rows(ctx, x, residual, cache, group, cos, sin, then_norm, accumulate)
+        qkv = ctx.scratch("attn_qkv", (t, (nq + 2 * nkv) * d), ctx.dtype)
         # 17..128 rows of a decode step: the q/k/v product and the preparation of its heads as two kernels, the
         # second adding up the sums of the product's K splits (no kernel of its own for that)
         together = (ctx.all_decode and self.b_qkv is None and ctx.dtype == torch.bfloat16 and t > self.PREPARE_INSIDE_ROWS
@@ -256,6 +288,57 @@ class GQAAttention(Part):
         else:
             ops.attention(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_slot, ctx.positions,
                           nq, self.scale, self.window or 0)
+        return linear(ctx, residual, out, self.w_o, accumulate=accumulate, then_norm=then_norm)
+
+    def _forward_whole_rows(self, ctx, x, residual, cache, group, cos, sin, then_norm, accumulate):
+        """The forms whose heads `qkv_norm_prep` prepares: one product for q, k, v (and the gate), the norms over the whole
+        projection, rotation and the write into the pages in one kernel, attention, the gate, the output projection."""
+        t, d, dv, nq, nkv = rows_of(x), self.head_dim, self.value_dim, self.num_heads, self.num_kv_heads
+        gate_at = (nq + nkv) * d + nkv * dv
+        qkv = ctx.scratch("attn_qkvg", (t, self.w_qkv.shape[0]), ctx.dtype)
+        linear(ctx, qkv, x, self.w_qkv)
+        ops.qkv_norm_prep(qkv, nq, nkv, d, dv, self.q_norm, self.k_norm, self.qk_norm_eps, cos, sin, cache.k_pages, cache.v_pages,
+                          group.slots, group.page_size)
+        out = ctx.scratch("attn_out", (t, nq * dv), ctx.dtype)
+        cores = dv == d and not self.keep_first and ops.attention_decode_supported(ctx.dtype, nq, nkv, d, group.page_size)
+        if cores and ctx.all_decode:
+            longest, bound = ctx.max_k, ctx.max_k_bound
+            if self.window is not None:
+                longest, bound = min(longest, self.window + 32), min(bound, self.window + 64)
+            splits = self._decode_splits(t * nkv, longest, bound, group.page_size)
+            part_o = part_ml = None
+            if splits > 1:
+                part_o = ctx.scratch("attn_part_o", (t, nq * splits * d), torch.float32)
+                part_ml = ctx.scratch("attn_part_ml", (t, nq * splits * 2), torch.float32)
+            ops.attention_decode(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_slot, ctx.positions,
+                                 nq, self.scale, self.window or 0, splits, part_o, part_ml, ctx.max_k_bound, None, form=1)
+        elif cores:
+            longest = ctx.max_k_bound if self.window is None else min(ctx.max_k_bound, self.window + 64)
+            singles = ctx.single_rows
+            if singles:
+                splits = self._decode_splits(singles * nkv, longest, ctx.max_k_bound, group.page_size)
+                part_o = part_ml = None
+                if splits > 1:
+                    part_o = ctx.scratch("attn_single_part_o", (singles, nq * splits * d), torch.float32)
+                    part_ml = ctx.scratch("attn_single_part_ml", (singles, nq * splits * 2), torch.float32)
+                ops.attention_decode(out[:singles], qkv[:singles], cache.k_pages, cache.v_pages, group.block_table, ctx.token_slot,
+                                     ctx.positions, nq, self.scale, self.window or 0, splits, part_o, part_ml, ctx.max_k_bound, None, form=1)
+            rest = ctx.memo.get("rows_after_singles")
+            if rest is None:
+                rest = ctx.memo["rows_after_singles"] = (ctx.token_slot[singles:], ctx.positions[singles:])
+            splits = self._prefill_splits(ctx.num_qblocks * nkv, longest, (t - singles) * nq * d, nq // nkv, t - singles)
+            part_o = part_ml = None
+            if splits > 1:
+                part_o = ctx.scratch("attn_part_o", (t - singles, nq * splits * d), torch.float32)
+                part_ml = ctx.scratch("attn_part_ml", (t - singles, nq * splits * 2), torch.float32)
+            ops.attention_prefill(out[singles:], qkv[singles:], cache.k_pages, cache.v_pages, group.block_table, rest[0], rest[1],
+                                  ctx.qblock_token0, ctx.qblock_count, nq, self.scale, self.window or 0, ctx.max_qblock, ctx.max_k_bound,
+                                  splits, part_o, part_ml, None)
+        else:
+            ops.attention(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_slot, ctx.positions, nq, self.scale,
+                          self.window or 0, self.keep_first)
+        if self.output_gate:
+            ops.sigmoid_gate(out, qkv[:, gate_at:gate_at + nq * dv])
         return linear(ctx, residual, out, self.w_o, accumulate=accumulate, then_norm=then_norm)
 
 

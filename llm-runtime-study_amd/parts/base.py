@@ -10,7 +10,7 @@ Roles and what each must provide:
   norm           forward(ctx, h, rows=None, count=None) -> x    h float32 [T, H] -> activation dtype; with `rows`
                                                         (int32 on the device) only the `count` rows listed there
   position       tables(ctx) -> (cos, sin) | None       float32 [T, rot/2] for this step's tokens
-  mixer          cache_need() -> PagedKVNeed | StateNeed | None
+  mixer          cache_need() -> PagedKVNeed | StateNeed | BothNeeds | None
                  forward(ctx, x, residual, cache)       adds its output into residual (float32)
   feed_forward   forward(ctx, x, residual)              adds its output into residual (float32)
   block          forward(ctx, h, cache)                 one layer: norms, mixer, feed-forward
@@ -34,7 +34,9 @@ Optional, each announced by a class attribute (a part without it is simply given
 
   handover_kind = "..."       block: forward(ctx, h, cache, given=None) returns something for the next block to start from
                               (the stream already rounded to the activation dtype, say), which the model passes on as
-                              `given` to the block that runs next if that one names the same kind, and to no other
+                              `given` to the block that runs next if that one names the same kind, and to no other;
+                              with `takes_next_norm = True` it is also told the first norm (`first_norm`) of the block that
+                              runs next, if that is of its kind: forward(ctx, h, cache, given=None, next_norm=None)
 
   wants_query_groups = True   mixer (a block passes it on): the step function cuts the tokens of a ragged step into
                               query groups for it: ctx.qblock_token0 / ctx.qblock_count [ctx.num_qblocks] list groups of
@@ -173,7 +175,8 @@ class TensorSpec:
     role: "matrix" ([out, in] projection), "embedding", "norm" (scale around 1), "bias";
     the random-weights mode draws each role differently.  dtype "float" follows the
     checkpoint (bfloat16 stays bfloat16, a tensor stored in 32-bit stays so); "int32"
-    marks integer tables.
+    marks integer tables.  A size of -1 stands for any size: the part reads it from the tensor it is given (random weights
+    cannot be drawn for such a shape: whoever wants them gives the size).
     """
 
     shape: tuple[int, ...]
@@ -194,6 +197,7 @@ class PagedKVNeed:
     window: int | None = None
     dtype: torch.dtype | None = None
     value_dim: int | None = None
+    keep_first: int = 0         # with a window: the first positions of a sequence stay visible for good, so their pages are never given back
 
 
 @dataclass(frozen=True)
@@ -202,6 +206,15 @@ class StateNeed:
 
     shape: tuple[int, ...]
     dtype: torch.dtype = torch.float32
+
+
+@dataclass(frozen=True)
+class BothNeeds:
+    """A mixer that keeps pages and a state of fixed size (two mixers side by side, one of each kind): the entry's LayerCache
+    then carries the group and pages of `paged` and the state rows of `state`."""
+
+    paged: PagedKVNeed
+    state: StateNeed
 
 
 class Part:

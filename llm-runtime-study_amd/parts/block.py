@@ -16,6 +16,12 @@ PostNormBlock: the sublayers read the stream itself and each norm is applied to 
 alpha is a constant of the model.  A sublayer writes into a float32 buffer of the step as for OutputNormBlock, and the norm's
 `scale_add_normed` does the rest in one kernel; a feed-forward that says `applies_sum_norm` is given norm and alpha and does
 it in the kernel that sums its output up.
+
+ParallelBlock: one norm, and both sublayers read its output; their sum, times a constant of the model, is added to the stream:
+    x = norm(h);  h = h + multiplier * (mixer(x) + feed_forward(x))      (the feed-forward may be absent)
+The mixer stores its output into a float32 buffer of the step, the feed-forward adds into it, and one kernel adds the buffer
+into the stream and leaves the next block's norm of the new stream beside it (`axpby` with a norm), which the model hands
+to the block that runs next if that is one of this kind.
 """
 
 from __future__ import annotations
@@ -290,3 +296,85 @@ class PostNormBlock(OutputNormBlock):
 
 
 register("block", "postnorm", PostNormBlock)
+
+
+class ParallelBlock(Part):
+    def __init__(self, mixer: PartSpec, norm: PartSpec, feed_forward: PartSpec | None = None, multiplier: float = 1.0, names: dict | None = None):
+        self.mixer = create("mixer", mixer)
+        self.norm = create("norm", norm)
+        self.feed_forward = None if feed_forward is None else create("feed_forward", feed_forward)
+        self.multiplier = float(multiplier)
+        if not getattr(self.mixer, "can_overwrite", False):
+            raise ValueError(f"the mixer of a parallel block must store its output (accumulate=False): {type(self.mixer).__name__} cannot")
+        self.names = {"mixer": "mixer", "feed_forward": "feed_forward", "norm": "norm"}
+        self.names.update(names or {})
+
+    def _children(self):
+        return [(self.names[k], getattr(self, k)) for k in ("norm", "mixer", "feed_forward") if getattr(self, k) is not None]
+
+    def tensors(self):
+        return {f"{prefix}.{name}": spec for prefix, part in self._children() for name, spec in part.tensors().items()}
+
+    def bind(self, weights, dtype):
+        for prefix, part in self._children():
+            part.bind(under(weights, prefix + "."), dtype)
+
+    def weight_bytes(self):
+        return sum(part.weight_bytes() for _, part in self._children())
+
+    def flops(self, tokens, pairs):
+        return sum(flops_of(part, tokens, pairs) for _, part in self._children())
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(part, "graph_safe", False) for _, part in self._children())
+
+    @property
+    def plan_safe(self) -> bool:
+        return all(getattr(part, "plan_safe", False) for _, part in self._children())
+
+    @property
+    def wants_query_groups(self) -> bool:
+        return getattr(self.mixer, "wants_query_groups", False)
+
+    # What a block of this kind hands the next one of its kind: (norm part, its normalised rows of the stream), made by the
+    # kernel that added this block's output into the stream; the next block uses them if its norm is the one named.
+    handover_kind = "normed_stream"
+    takes_next_norm = True
+
+    @property
+    def first_norm(self):
+        return self.norm
+
+    def forward(self, ctx, h, cache, given=None, next_norm=None):
+        if given is not None and given[0] is self.norm:
+            x = given[1]
+        else:
+            x = self.norm.forward(ctx, h)
+        y = ctx.scratch("sublayer_out", tuple(h.shape), torch.float32)
+        self.mixer.forward(ctx, x, y, cache, accumulate=False)
+        if self.feed_forward is not None:
+            self.feed_forward.forward(ctx, x, y)
+        parameters = getattr(next_norm, "rms_parameters", None)
+        if parameters is None:
+            ops.axpby(h, h, 1.0, y, self.multiplier)
+            return None
+        weight, eps = parameters()
+        turn = ctx.memo["normed_stream_turn"] = 1 - ctx.memo.get("normed_stream_turn", 0)     # not the buffer this block's x lies in
+        normed = ctx.scratch(f"stream_normed{turn}", tuple(h.shape), ctx.dtype)
+        ops.axpby(h, h, 1.0, y, self.multiplier, weight if weight.dtype == torch.float32 else self._weight_f32(next_norm, weight), eps, normed)
+        return (next_norm, normed)
+
+    @staticmethod
+    def _weight_f32(norm, weight):
+        """The norm's weight in float32 (made once and kept on the norm part)."""
+        kept = getattr(norm, "_weight_f32", None)
+        if kept is None or kept.device != weight.device:
+            kept = norm._weight_f32 = weight.float().contiguous()
+        return kept
+
+
+register("block", "parallel", ParallelBlock)

@@ -11,6 +11,12 @@ For a token with input x, per head h (key group h // (heads / kv_heads), as in g
 `unit(z) = z / sqrt(sum(z^2) + 1e-6)`.  The gates, the unit norms, the state and the read-out are float32 in
 every run; the projections that feed them are written in float32 too.
 
+`channel_decay` (with `decay_rank`, `gate_rank`): the decay is one number per head and key channel, multiplying the rows of S,
+    g = exp(-exp(A_log_h) * softplus(W_a2 (W_a1 x) + dt_bias))  laid out heads x head_dim, dt_bias of that size,
+and the output gate is sigmoid(W_g2 (W_g1 x)) laid out heads x value_dim; W_a1 and W_g1 are stacked behind q, k, v and the step
+size, the second matrices are applied in float32 inside the recurrence's kernels.  A rank of None is read from the checkpoint's
+tensors when they are bound.
+
 All six input projections are one stacked product.  What a request keeps between steps is one float32 row: the
 matrices of all heads, then the convolution's last taps - 1 inputs of every channel (`StateNeed`); the cache
 manager hands out the rows, clears a row at admission and the kernels find a request's row by its slot.
@@ -37,7 +43,8 @@ class GatedDeltaRule(Part):
     plan_safe = True
     can_overwrite = True
 
-    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, conv_taps: int, norm_eps: float):
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, conv_taps: int, norm_eps: float,
+                 channel_decay: bool = False, decay_rank: int | None = None, gate_rank: int | None = None):
         for name, value in (("hidden_size", hidden_size), ("num_heads", num_heads), ("num_kv_heads", num_kv_heads), ("head_dim", head_dim),
                             ("value_dim", value_dim), ("conv_taps", conv_taps)):
             if value <= 0:
@@ -52,10 +59,20 @@ class GatedDeltaRule(Part):
         self.head_dim, self.value_dim, self.conv_taps, self.norm_eps = head_dim, value_dim, conv_taps, norm_eps
         self.channels = 2 * num_kv_heads * head_dim + num_heads * value_dim          # what passes the convolution: q, k, v
         self.columns = self.channels + num_heads * value_dim + 2 * num_heads          # ... and the output gate, step size, decay input
-        self.w_in = self.w_o = self.conv = self.a_log = self.dt_bias = self.norm = None
+        if not channel_decay and (decay_rank is not None or gate_rank is not None):
+            raise ValueError("decay_rank and gate_rank belong to channel_decay")
+        for name, value in (("decay_rank", decay_rank), ("gate_rank", gate_rank)):
+            if value is not None and value <= 0:
+                raise ValueError(f"{name} must be positive when given, got {value}")
+        self.channel_decay, self.decay_rank, self.gate_rank = channel_decay, decay_rank, gate_rank
+        self.w_in = self.w_o = self.conv = self.a_log = self.dt_bias = self.norm = self.decay_up = self.gate_up = None
 
     def _projections(self):
         qk, v = self.num_kv_heads * self.head_dim, self.num_heads * self.value_dim
+        if self.channel_decay:
+            # a rank that is not given is whatever the checkpoint holds: -1 in a shape stands for any size
+            return (("q_proj", qk), ("k_proj", qk), ("v_proj", v), ("b_proj", self.num_heads), ("a1_proj", self.decay_rank or -1),
+                    ("g1_proj", self.gate_rank or -1))
         return (("q_proj", qk), ("k_proj", qk), ("v_proj", v), ("g_proj", v), ("b_proj", self.num_heads), ("a_proj", self.num_heads))
 
     def tensors(self):
@@ -63,7 +80,10 @@ class GatedDeltaRule(Part):
         for name, width in self._projections()[:3]:
             specs[f"{name[0]}_conv.weight"] = TensorSpec((width, self.conv_taps))
         specs["A_log"] = TensorSpec((self.num_heads,), role="bias")
-        specs["dt_bias"] = TensorSpec((self.num_heads,), role="bias")
+        specs["dt_bias"] = TensorSpec((self.num_heads * self.head_dim if self.channel_decay else self.num_heads,), role="bias")
+        if self.channel_decay:
+            specs["a2_proj.weight"] = TensorSpec((self.num_heads * self.head_dim, self.decay_rank or -1))
+            specs["g2_proj.weight"] = TensorSpec((self.num_heads * self.value_dim, self.gate_rank or -1))
         specs["norm.weight"] = TensorSpec((self.value_dim,), role="norm")
         specs["o_proj.weight"] = TensorSpec((self.hidden_size, self.num_heads * self.value_dim))
         return specs
@@ -78,6 +98,14 @@ class GatedDeltaRule(Part):
         self.a_log, self.dt_bias = weights["A_log"].float().contiguous(), weights["dt_bias"].float().contiguous()
         self.norm = weights["norm.weight"].float().contiguous()
         self.w_o = weights["o_proj.weight"].to(dtype).contiguous()
+        if self.channel_decay:
+            # the second matrices by columns, so that neighbouring lanes read neighbouring values: [rank, outputs] float32
+            self.decay_up = weights["a2_proj.weight"].float().t().contiguous()
+            self.gate_up = weights["g2_proj.weight"].float().t().contiguous()
+            first = {name: weights[f"{name}.weight"].shape[0] for name in ("a1_proj", "g1_proj")}
+            if (first["a1_proj"], first["g1_proj"]) != (self.decay_up.shape[0], self.gate_up.shape[0]):
+                raise ValueError(f"the two matrices of a low-rank input disagree: {first} against {self.decay_up.shape[0]} and {self.gate_up.shape[0]}")
+            self.decay_rank, self.gate_rank = self.decay_up.shape[0], self.gate_up.shape[0]
 
     def weight_bytes(self):
         return (self.w_in.numel() + self.w_o.numel()) * self.w_o.element_size()
@@ -103,6 +131,13 @@ class GatedDeltaRule(Part):
         qkv = ctx.scratch("delta_qkv", (t, self.channels), torch.float32)
         gates = ctx.scratch("delta_gates", (t, 2 * self.num_heads), torch.float32)
         raw = ctx.scratch("delta_read_out", (t, self.num_heads * self.value_dim), torch.float32)
+        if self.channel_decay:
+            decays = ctx.scratch("delta_decays", (t, self.num_heads * self.head_dim), torch.float32)
+            ops.delta_rule_channels(out, proj, cache.state, ctx.token_request, ctx.cu_seqlens_q, ctx.slot_ids, ctx.R, self.conv, self.num_kv_heads,
+                                    self.num_heads, self.head_dim, self.value_dim, self.a_log, self.dt_bias, self.norm, self.norm_eps, qkv, gates, raw,
+                                    self.decay_up, decays, self.gate_up)
+            linear(ctx, residual, out, self.w_o, accumulate=accumulate)
+            return None
         ops.delta_rule(out, proj, cache.state, ctx.token_request, ctx.cu_seqlens_q, ctx.slot_ids, ctx.R, self.conv, self.num_kv_heads,
                        self.num_heads, self.head_dim, self.value_dim, self.a_log, self.dt_bias, self.norm, self.norm_eps, qkv, gates, raw)
         linear(ctx, residual, out, self.w_o, accumulate=accumulate)

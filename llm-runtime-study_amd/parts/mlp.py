@@ -1,4 +1,5 @@
-"""SwiGLU feed-forward: down(silu(gate(x)) * up(x)), three bias-free projections.
+"""Feed-forwards.  SwiGLU: down(silu(gate(x)) * up(x)), three bias-free projections; DenseMLP (at the end of the file):
+down(act(up(x))), two bias-free projections with an activation between them.
 
 Reference mini_llm/nn/mlp.py:80-87.  gate and up are stacked into one [2I, H] matrix when
 the weights are bound, so one product feeds the gated activation; the down projection adds
@@ -64,3 +65,42 @@ class SwiGLU(Part):
 
 
 register("feed_forward", "swiglu", SwiGLU)
+
+
+class DenseMLP(Part):
+    """down(act(up(x))): two bias-free projections, `activation` between them: "gelu" (the exact one, 0.5 z (1 + erf(z / sqrt 2))),
+    "gelu_tanh", "silu" or "relu" (kernels/ops.py, ACTIVATIONS).  The down projection adds into the float32 rows it is given, or
+    stores into them with `accumulate=False`."""
+
+    graph_safe = True
+    plan_safe = True
+    can_overwrite = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "gelu"):
+        if hidden_size <= 0 or intermediate_size <= 0:
+            raise ValueError("hidden_size and intermediate_size must be positive")
+        if activation not in ops.ACTIVATIONS:
+            raise ValueError(f"unknown activation {activation!r}; known: {', '.join(ops.ACTIVATIONS)}")
+        self.hidden_size, self.intermediate_size, self.activation = hidden_size, intermediate_size, activation
+        self.up = self.down = None
+
+    def tensors(self):
+        return {"up_proj.weight": TensorSpec((self.intermediate_size, self.hidden_size)),
+                "down_proj.weight": TensorSpec((self.hidden_size, self.intermediate_size))}
+
+    def bind(self, weights, dtype):
+        self.up = weights["up_proj.weight"].to(dtype).contiguous()
+        self.down = weights["down_proj.weight"].to(dtype).contiguous()
+
+    def weight_bytes(self):
+        return (self.up.numel() + self.down.numel()) * self.down.element_size()
+
+    def forward(self, ctx, x, residual, then_norm=None, accumulate: bool = True):
+        t = rows_of(x)
+        act = ctx.scratch("ffn_act", (t, self.intermediate_size), ctx.dtype)
+        linear(ctx, act, x, self.up)
+        ops.activation(act, act, self.activation)
+        return linear(ctx, residual, act, self.down, accumulate=accumulate, then_norm=then_norm)
+
+
+register("feed_forward", "dense_mlp", DenseMLP)

@@ -18,18 +18,25 @@ from .base import Part, register
 
 
 class RotaryHalfSplit(Part):
-    def __init__(self, rotary_dim: int, theta: float):
+    """Pairs (i, i + rotary_dim/2) turned by position * theta^(-2i/rotary_dim) / factor; `factor` (linear scaling of the
+    positions: every frequency divided by it) is 1 unless given."""
+
+    def __init__(self, rotary_dim: int, theta: float, factor: float = 1.0):
         if rotary_dim <= 0 or rotary_dim % 2 != 0:
             raise ValueError(f"rotary_dim must be a positive even integer, got {rotary_dim}")
         if theta <= 0:
             raise ValueError(f"theta must be positive, got {theta}")
-        self.rotary_dim, self.theta = rotary_dim, theta
+        if not factor > 0:
+            raise ValueError(f"factor must be positive, got {factor}")
+        self.rotary_dim, self.theta, self.factor = rotary_dim, theta, float(factor)
         dims = torch.arange(0, rotary_dim, 2, dtype=torch.float32)
         self._inv_freq_host = 1.0 / (theta ** (dims / rotary_dim))
+        if self.factor != 1.0:
+            self._inv_freq_host = self._inv_freq_host / self.factor
         self._inv_freq = None
 
     def key(self):
-        return ("rope_half", self.rotary_dim, self.theta)
+        return ("rope_half", self.rotary_dim, self.theta, self.factor)
 
     def tables(self, ctx):
         """cos and sin [T, rotary_dim/2] float32 for this step's positions (made once per step)."""
@@ -38,8 +45,9 @@ class RotaryHalfSplit(Part):
             if self._inv_freq is None or self._inv_freq.device != ctx.positions.device:
                 self._inv_freq = self._inv_freq_host.to(ctx.positions.device)
             half = self.rotary_dim // 2
-            cos = ctx.scratch(f"rope_cos_{self.rotary_dim}_{self.theta}", (ctx.T, half), torch.float32)
-            sin = ctx.scratch(f"rope_sin_{self.rotary_dim}_{self.theta}", (ctx.T, half), torch.float32)
+            tag = f"{self.rotary_dim}_{self.theta}" + ("" if self.factor == 1.0 else f"_{self.factor}")
+            cos = ctx.scratch(f"rope_cos_{tag}", (ctx.T, half), torch.float32)
+            sin = ctx.scratch(f"rope_sin_{tag}", (ctx.T, half), torch.float32)
             ops.rope_table(cos, sin, ctx.positions, self._inv_freq)
             cached = ctx.memo[self.key()] = (cos, sin)
         return cached

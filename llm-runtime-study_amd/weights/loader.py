@@ -51,7 +51,8 @@ def validate(checkpoint: Checkpoint, expected: Mapping[str, TensorSpec], archite
         errors.append("unexpected tensors: " + ", ".join(unexpected))
     for name in sorted(expected.keys() & actual.keys()):
         spec, info = expected[name], actual[name]
-        if info.shape != tuple(spec.shape):
+        # -1 in an expected shape stands for any size (a part that reads that size from the checkpoint when it binds)
+        if len(info.shape) != len(spec.shape) or any(want != -1 and want != got for want, got in zip(spec.shape, info.shape)):
             errors.append(f"shape mismatch for {name}: expected {tuple(spec.shape)}, got {info.shape}")
         if spec.dtype == "int32":
             if info.dtype not in INT_DTYPES:
