@@ -30,10 +30,15 @@ from .safetensors_io import write_safetensors
 TORCH_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32, "float16": torch.float16}
 
 
-def _draw(spec: TensorSpec, init: str, generator, device="cpu") -> torch.Tensor:
+def _draw(spec: TensorSpec, init: str, generator, device="cpu", free_size: int | None = None) -> torch.Tensor:
+    shape = tuple(spec.shape)
+    if -1 in shape:          # a size the part reads from its checkpoint: the caller of a random model chooses it
+        if free_size is None:
+            raise ValueError(f"a tensor of shape {shape} has a size that only a checkpoint gives: pass free_size")
+        shape = tuple(free_size if size == -1 else size for size in shape)
     if spec.dtype == "int32":
-        return torch.zeros(spec.shape, dtype=torch.int32, device=device)
-    noise = torch.randn(spec.shape, generator=generator, device=device, dtype=torch.float32)
+        return torch.zeros(shape, dtype=torch.int32, device=device)
+    noise = torch.randn(shape, generator=generator, device=device, dtype=torch.float32)
     if init == "normal":
         return 1.0 + 0.02 * noise if spec.role == "norm" else 0.02 * noise
     if init == "scaled":
@@ -43,36 +48,38 @@ def _draw(spec: TensorSpec, init: str, generator, device="cpu") -> torch.Tensor:
             return 0.1 * noise
         if spec.role == "embedding":
             return noise
-        return noise / float(spec.shape[-1]) ** 0.5
+        return noise / float(shape[-1]) ** 0.5
     raise ValueError(f"unknown init {init!r}; expected 'normal' or 'scaled'")
 
 
-def random_tensors(expected: dict[str, TensorSpec], seed: int, dtype: torch.dtype, init: str = "normal") -> dict[str, torch.Tensor]:
+def random_tensors(expected: dict[str, TensorSpec], seed: int, dtype: torch.dtype, init: str = "normal",
+                   free_size: int | None = None) -> dict[str, torch.Tensor]:
+    """free_size: what every size that a part leaves to its checkpoint (-1 in a TensorSpec's shape) is drawn as."""
     generator = torch.Generator().manual_seed(seed)
-    return {name: _draw(expected[name], init, generator).to(torch.int32 if expected[name].dtype == "int32" else dtype)
+    return {name: _draw(expected[name], init, generator, free_size=free_size).to(torch.int32 if expected[name].dtype == "int32" else dtype)
             for name in sorted(expected) if not expected[name].optional}
 
 
-def write_model_dir(config, seed: int, model_dir, init: str = "normal") -> Path:
+def write_model_dir(config, seed: int, model_dir, init: str = "normal", free_size: int | None = None) -> Path:
     """Write config.json and model.safetensors for `config` (a typed configuration)."""
     model_dir = Path(model_dir)
     model_dir.mkdir(parents=True, exist_ok=True)
     spec = spec_for(config)
     expected = DecoderModel(spec).tensors()
-    tensors = random_tensors(expected, seed, TORCH_DTYPES[spec.checkpoint_dtype], init)
+    tensors = random_tensors(expected, seed, TORCH_DTYPES[spec.checkpoint_dtype], init, free_size)
     (model_dir / "config.json").write_text(json.dumps(config.to_json_dict(), indent=2) + "\n")
     write_safetensors(model_dir / "model.safetensors", tensors, {"seed": seed, "init": init})
     return model_dir
 
 
-def device_weights(model: DecoderModel, seed: int, dtype: torch.dtype, device, init: str = "normal") -> LazyTensors:
+def device_weights(model: DecoderModel, seed: int, dtype: torch.dtype, device, init: str = "normal", free_size: int | None = None) -> LazyTensors:
     expected = model.tensors()
     names = [name for name in sorted(expected) if not expected[name].optional]
     place = {name: index for index, name in enumerate(names)}
 
     def draw(name: str) -> torch.Tensor:
         generator = torch.Generator(device=device).manual_seed((seed << 20) + place[name])
-        return _draw(expected[name], init, generator, device).to(torch.int32 if expected[name].dtype == "int32" else dtype)
+        return _draw(expected[name], init, generator, device, free_size).to(torch.int32 if expected[name].dtype == "int32" else dtype)
 
     return LazyTensors(names, draw)
 
@@ -88,10 +95,11 @@ def main(argv=None) -> int:
     parser.add_argument("--seed", type=int, default=0)
     parser.add_argument("--out", type=Path, required=True)
     parser.add_argument("--init", choices=("normal", "scaled"), default="normal")
+    parser.add_argument("--free-size", type=int, default=None, help="for sizes that only a checkpoint gives (the rank of a low-rank input)")
     args = parser.parse_args(argv)
     path = args.config / "config.json" if args.config.is_dir() else args.config
     config = config_from_dict(json.loads(path.read_text()))
-    write_model_dir(config, args.seed, args.out, args.init)
+    write_model_dir(config, args.seed, args.out, args.init, args.free_size)
     print(f"wrote {args.out}/config.json and model.safetensors")
     return 0
 
