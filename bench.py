@@ -3,6 +3,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 2048] [--layers L] [--shape 8b|14b|32b]
     python bench.py --design nobodra [--shape 8b] [--layers 8] ...     # the Nobodra design at the shape's layer sizes, beside the shape itself
     python bench.py --design napizen [--shape 8b] [--layers 8] ...     # the same for the Napizen design
+    python bench.py --design kaposun [--shape 8b] [--layers 8] ...     # the same for the Kaposun design
 
 A step is one decode step of the whole engine (scheduler, step function, sampling) at the
 given batch; `value` is decoded tokens per second.  The same line carries the prefill rate
@@ -27,7 +28,7 @@ if str(ROOT) not in sys.path:
 HBM_PEAK = 8.0e12
 FLOP_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
 
-from llm_runtime_study_amd.benchmarks.shapes import QWEN3_8B, SHAPES, napizen_like, nobodra_like  # noqa: E402  (layer sizes of the 8B, 14B and 32B models)
+from llm_runtime_study_amd.benchmarks.shapes import QWEN3_8B, SHAPES, kaposun_like, napizen_like, nobodra_like  # noqa: E402  (layer sizes of the 8B, 14B and 32B models)
 
 FULL_LAYERS = QWEN3_8B["num_hidden_layers"]
 BENCHMARK_CONTEXT = 4096      # tokens a request's cache can hold at the least: the benchmark context of the 8B configuration
@@ -47,8 +48,8 @@ def parse_args():
     parser.add_argument("--num-pages", type=int, default=None, help="pages of the cache pool (default: max-seq-len tokens for every request of the largest batch)")
     parser.add_argument("--shape", choices=tuple(SHAPES), default="8b", help="layer sizes: Qwen3-8B (default), 14B or 32B")
     parser.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (reported in config)")
-    parser.add_argument("--design", choices=("qwen3", "nobodra", "napizen"), default="qwen3",
-                        help="nobodra, napizen: measure that design at the shape's layer sizes (8 layers unless --layers says otherwise) and, beside it, the shape itself with as many layers")
+    parser.add_argument("--design", choices=("qwen3", "nobodra", "napizen", "kaposun"), default="qwen3",
+                        help="nobodra, napizen, kaposun: measure that design at the shape's layer sizes (8 layers unless --layers says otherwise) and, beside it, the shape itself with as many layers")
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
     parser.add_argument("--temperature", type=float, default=0.0, help="draw the tokens at this temperature instead of taking the largest logit (reported in config)")
@@ -190,7 +191,7 @@ def step_bytes(engine, batch: int, mean_context: float) -> float:
     that the batch's tokens choose between them: experts * (1 - (1 - top / experts) ** batch) of them on average."""
     import math
 
-    from llm_runtime_study_amd.parts import PagedKVNeed, StateNeed
+    from llm_runtime_study_amd.parts import BothNeeds, PagedKVNeed, StateNeed
 
     model, total = engine.model, 0.0
     for entry, need in zip(model.spec.schedule, model.cache_needs()):
@@ -200,12 +201,13 @@ def step_bytes(engine, batch: int, mean_context: float) -> float:
         if ff is not None and hasattr(ff, "num_experts"):
             hit = ff.num_experts * (1.0 - (1.0 - ff.top / ff.num_experts) ** batch)
             total += (hit - ff.top) * (3 if getattr(ff, "gated", False) else 2) * ff.hidden_size * ff.intermediate_size * ff.up.element_size()
-        if isinstance(need, PagedKVNeed):
-            held = mean_context if need.window is None else min(mean_context, need.window)
-            kept = need.head_dim + (need.head_dim if need.value_dim is None else need.value_dim)
-            total += batch * held * need.num_kv_heads * kept * (2 if engine.dtype == torch_bfloat16() else 4)
-        elif isinstance(need, StateNeed):
-            total += 2 * batch * math.prod(need.shape) * 4
+        for need in ((need.paged, need.state) if isinstance(need, BothNeeds) else (need,)):
+            if isinstance(need, PagedKVNeed):
+                held = mean_context if need.window is None else min(mean_context, need.window + need.keep_first)
+                kept = need.head_dim + (need.head_dim if need.value_dim is None else need.value_dim)
+                total += batch * held * need.num_kv_heads * kept * (2 if engine.dtype == torch_bfloat16() else 4)
+            elif isinstance(need, StateNeed):
+                total += 2 * batch * math.prod(need.shape) * 4
     return total + model.head.numel() * model.head.element_size()
 
 
@@ -238,7 +240,7 @@ def measure_design(args, config, dtype_name: str, max_seq_len: int, max_batch: i
 
 
 def design_main(args) -> int:
-    """--design nobodra | napizen: the design at the shape's layer sizes, and the shape itself with as many layers, one after the other."""
+    """--design nobodra | napizen | kaposun: the design at the shape's layer sizes, and the shape itself with as many layers, one after the other."""
     import gc
 
     import torch
@@ -250,8 +252,8 @@ def design_main(args) -> int:
     max_batch = args.batch if args.no_points else max(args.batch, 64)
     max_seq_len = args.max_seq_len or max(BENCHMARK_CONTEXT, args.context + args.steps + warmup_room(args.warmup, max(args.decode_steps_per_launch, 1))
                                           + decode_lead(max_batch, args.context, max(2048, args.prefill_tokens)) + max_batch + 64, args.prefill_tokens + 1)
-    name = {"nobodra": "Nobodra", "napizen": "Napizen"}[args.design]
-    raw = (nobodra_like if args.design == "nobodra" else napizen_like)(SHAPES[args.shape], layers)
+    name = {"nobodra": "Nobodra", "napizen": "Napizen", "kaposun": "Kaposun"}[args.design]
+    raw = {"nobodra": nobodra_like, "napizen": napizen_like, "kaposun": kaposun_like}[args.design](SHAPES[args.shape], layers)
     mine = measure_design(args, config_from_dict(raw), dtype_name, max_seq_len, max_batch)
     gc.collect()
     torch.cuda.empty_cache()
@@ -264,6 +266,7 @@ def design_main(args) -> int:
         "data": "synthetic (seeded uniform random token ids, random weights N(0, 0.02))",
         "config": {"model": f"{name} at Qwen3-{args.shape.upper()} layer sizes", "layers": layers, "width": raw["width"], "layer_kinds": [layer["type"] for layer in raw["layers"]],
                    "mixer": raw["layers"][-1]["mixer"] if layers >= 4 else raw["layers"][0]["mixer"], "first_mixer": raw["layers"][0]["mixer"],
+                   **({"third_mixer": raw["layers"][2]["mixer"]} if args.design == "kaposun" and layers >= 3 else {}),
                    "mlp": [raw["layers"][0]["mlp"], raw["layers"][-1]["mlp"]],
                    "global_batch": args.batch, "seq_len": args.context, "max_seq_len": max_seq_len, "prefill_tokens": args.prefill_tokens, "parallelism": "single GPU"},
         args.design: mine,

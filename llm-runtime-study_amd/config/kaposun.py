@@ -213,6 +213,12 @@ class KaposunConfig:
         start, stop, times = self.loop
         return tuple(range(start)) + tuple(range(start, stop)) * times + tuple(range(stop, count))
 
+    @property
+    def random_rank(self) -> int:
+        """The rank of the delta rule's low-rank inputs (decay, output gate) when weights are drawn at random: a checkpoint's
+        tensors give it otherwise, config.json does not."""
+        return max(4, self.width // 32)
+
     def validate_context_length(self, max_seq_len: int) -> None:
         if not 0 < max_seq_len <= MAX_POSITIONS:
             raise ConfigError(f"max_seq_len must be within 1..{MAX_POSITIONS}, got {max_seq_len}")

@@ -234,7 +234,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_bf16_kernel(
     const bf16* __restrict__ q, int q_stride, bf16* __restrict__ k_pages,
     bf16* __restrict__ v_pages, const int* __restrict__ block_table, int table_stride,
     const int* __restrict__ token_request, const int* __restrict__ positions, int nq, int nkv,
-    int page_size, float scale, int window, int splits, DecodePrep prep) {
+    int page_size, float scale, int window, int splits, int slots, DecodePrep prep) {
   constexpr int DS = D / 32, DB = D / 16, THREADS = WAVES * 64;
   __shared__ float sm_m[WAVES][16], sm_l[WAVES][16];
   __shared__ float sm_o[WAVES][D][16];
@@ -473,10 +473,10 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_bf16_kernel(
       total += sm_l[w][h] * weight;
     }
     const int head = kvh * group + h;
-    if (splits == 1) {
+    if (slots <= 1) {
       out[(int64_t)token * out_stride + (int64_t)head * D + dim] = (bf16)(acc / total);
     } else {
-      const int64_t slot = ((int64_t)token * nq + head) * splits + split;
+      const int64_t slot = ((int64_t)token * nq + head) * slots + split;
       part_o[slot * D + dim] = acc;
       if (dim == 0) {
         part_ml[slot * 2] = top;
@@ -571,21 +571,94 @@ __global__ __launch_bounds__(256) void attention_merge_wide_kernel(bf16* __restr
 static void launch_attention_merge(bf16* out, int out_stride, const float* part_o, const float* part_ml, int tokens, int nq, int d,
                                    int splits, hipStream_t s) {
   const bool wide = tokens >= 64 && d % 4 == 0 && out_stride % 4 == 0 && (uintptr_t)out % 8 == 0 && (uintptr_t)part_o % 16 == 0 &&
-                    (uintptr_t)part_ml % 8 == 0 && (splits == 2 || splits == 3 || splits == 4 || splits == 8);
+                    (uintptr_t)part_ml % 8 == 0 && (splits == 2 || splits == 3 || splits == 4 || splits == 5 || splits == 8 || splits == 9);
   if (wide) {
     const int64_t quads = (int64_t)tokens * nq * (d / 4);
     const int blocks = (int)((quads + 255) / 256);
     if (splits == 2) attention_merge_wide_kernel<2><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d);
     else if (splits == 3) attention_merge_wide_kernel<3><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d);
     else if (splits == 4) attention_merge_wide_kernel<4><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d);
+    else if (splits == 5) attention_merge_wide_kernel<5><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d);
+    else if (splits == 9) attention_merge_wide_kernel<9><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d);
     else attention_merge_wide_kernel<8><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d);
   } else {
     attention_merge_kernel<<<dim3(tokens, nq), d < 64 ? 64 : d, 0, s>>>(out, out_stride, part_o, part_ml, nq, d, splits);
   }
 }
 
+// The share of a sequence's kept first positions in a windowed attention: for every (token, head) the keys at positions
+// below min(keep_first, lo), lo = pos - window + 1 being the window's first position (none while the window still reaches
+// the start), as one more partial result beside those of the window's splits: unnormalised sums against a maximum, in the
+// form attention_merge_kernel adds up (slot `slots - 1` of part_o [tokens, nq, slots, d] and part_ml [tokens, nq, slots, 2]).
+// A wave per (token, head), a lane for every 64th dim; the kept keys are few, and every one is a row of d values.
+__global__ __launch_bounds__(WAVE) void attention_kept_bf16_kernel(
+    const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
+    const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_request,
+    const int* __restrict__ positions, int nq, int nkv, int d, int page_size, float scale, int window, int keep_first,
+    int slots, float* __restrict__ part_o, float* __restrict__ part_ml) {
+  constexpr int PER_LANE = 4;                                     // heads of up to 256 dims
+  const int token = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const int kvh = head / (nq / nkv);
+  const int pos = positions[token];
+  const int lo = pos - window + 1;
+  const int kept = lo > 0 ? (keep_first < lo ? keep_first : lo) : 0;
+  const int64_t slot = ((int64_t)token * nq + head) * slots + (slots - 1);
+  const float scale2 = scale * 1.4426950408889634f;
+  const int* table = block_table + (int64_t)token_request[token] * table_stride;
+  float qv[PER_LANE], acc[PER_LANE];
+#pragma unroll
+  for (int n = 0; n < PER_LANE; ++n) {
+    const int dim = lane + n * WAVE;
+    qv[n] = dim < d ? (float)q[(int64_t)token * q_stride + (int64_t)head * d + dim] : 0.f;
+    acc[n] = 0.f;
+  }
+  float top = -INFINITY, total = 0.f;
+  for (int key = 0; key < kept; ++key) {
+    const int64_t page = table[key / page_size];
+    const int off = key % page_size;
+    const bf16* kp = k_pages + ((page * nkv + kvh) * page_size + off) * (int64_t)d;
+    const bf16* vp = v_pages + (page * nkv + kvh) * (int64_t)d * page_size + off;
+    float dot = 0.f, vv[PER_LANE];
+#pragma unroll
+    for (int n = 0; n < PER_LANE; ++n) {
+      const int dim = lane + n * WAVE;
+      dot += dim < d ? qv[n] * (float)kp[dim] : 0.f;
+      vv[n] = dim < d ? (float)vp[(int64_t)dim * page_size] : 0.f;
+    }
+#pragma unroll
+    for (int step = 1; step < WAVE; step *= 2) dot += __shfl_xor(dot, step, WAVE);
+    const float score = dot * scale2;
+    const float new_top = fmaxf(top, score);
+    const float keep = top == -INFINITY ? 0.f : fast_exp2(top - new_top);
+    const float weight = fast_exp2(score - new_top);
+    total = total * keep + weight;
+#pragma unroll
+    for (int n = 0; n < PER_LANE; ++n) acc[n] = acc[n] * keep + weight * vv[n];
+    top = new_top;
+  }
+#pragma unroll
+  for (int n = 0; n < PER_LANE; ++n) {
+    const int dim = lane + n * WAVE;
+    if (dim < d) part_o[slot * d + dim] = acc[n];
+  }
+  if (lane == 0) {
+    part_ml[slot * 2] = top;
+    part_ml[slot * 2 + 1] = total;
+  }
+}
+
+static void launch_attention_kept(const bf16* q, int q_stride, const bf16* k_pages, const bf16* v_pages, const int* block_table,
+                                  int table_stride, const int* token_request, const int* positions, int tokens, int nq, int nkv, int d,
+                                  int page_size, float scale, int window, int keep_first, int slots, float* part_o, float* part_ml,
+                                  hipStream_t s) {
+  attention_kept_bf16_kernel<<<dim3(tokens, nq), WAVE, 0, s>>>(q, q_stride, k_pages, v_pages, block_table, table_stride, token_request,
+                                                               positions, nq, nkv, d, page_size, scale, window, keep_first, slots, part_o,
+                                                               part_ml);
+}
+
 // Decode step in bf16: one query token per request.  part_o [tokens, nq, splits, d] and part_ml
-// [tokens, nq, splits, 2] float32 are needed when splits > 1.  Returns an error for shapes the
+// [tokens, nq, splits, 2] float32 are needed when splits > 1; with keep_first (a window's kept first positions, see
+// attention_kept_bf16_kernel) they hold one partial result more and are always needed.  Returns an error for shapes the
 // matrix-core kernel does not take (the caller then uses lrs_attention).
 // prepare != 0: q points at the raw rows [q heads | kv_columns k heads | kv_columns v heads] of the
 // q/k/v product and the kernel does the work of lrs_qk_prep as well (rotation over the whole head
@@ -594,14 +667,16 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
                                  int q_stride, void* k_pages, void* v_pages,
                                  const int* block_table, int table_stride, const int* token_request,
                                  const int* positions, int tokens, int max_context, int nq, int nkv, int d,
-                                 int page_size, float scale, int window, int splits, int form, int prepare,
+                                 int page_size, float scale, int window, int keep_first, int splits, int form, int prepare,
                                  const void* q_weight, const void* k_weight, int w_dtype, float eps,
                                  const float* cosv, const float* sinv, int kv_columns, void* stream) {
   LRS_REQUIRE(tokens > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_decode: bad sizes tokens=%d nq=%d nkv=%d", tokens, nq, nkv);
   LRS_REQUIRE(nq / nkv <= 16, "attention_decode: %d query heads per kv head, at most 16 fit a tile", nq / nkv);
   LRS_REQUIRE(page_size % 16 == 0, "attention_decode: page size %d is not a multiple of 16", page_size);
-  LRS_REQUIRE(splits >= 1 && (splits == 1 || (part_o && part_ml)), "attention_decode: splits=%d needs partial buffers", splits);
-  LRS_REQUIRE(window >= 0, "attention_decode: window must be >= 0 (0 = none)");
+  LRS_REQUIRE(window >= 0 && keep_first >= 0 && (keep_first == 0 || (window > 0 && !prepare)),
+              "attention_decode: kept first positions (%d) need a window and prepared heads", keep_first);
+  const int slots = splits + (keep_first > 0 ? 1 : 0);          // the kept keys' share is one more partial result
+  LRS_REQUIRE(splits >= 1 && (slots == 1 || (part_o && part_ml)), "attention_decode: %d partial results need their buffers", slots);
   LRS_REQUIRE(form >= 0 && form <= 2, "attention_decode: form must be 0, 1 or 2, got %d", form);
   LRS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0, "attention_decode: q rows must be 16-byte aligned");
   dim3 grid(splits, nkv, tokens);
@@ -626,7 +701,7 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
   // tile on the way while it works (heads of 192 dims have no registers for that and stay with 0)
 #define ARGS                                                                                                 \
   (bf16*)out, out_stride, part_o, part_ml, (const bf16*)q, q_stride, (bf16*)k_pages, (bf16*)v_pages, block_table, \
-      table_stride, token_request, positions, nq, nkv, page_size, scale, window, splits, prep
+      table_stride, token_request, positions, nq, nkv, page_size, scale, window, splits, slots, prep
 #define LAUNCH_PREP(D, PREP)                                                                                 \
   do {                                                                                                       \
     if (form == 2 && D <= 128) attention_decode_bf16_kernel<D, PREP, 8, (D <= 128)><<<grid, 512, table_lds, s>>>(ARGS); \
@@ -650,8 +725,13 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
 #undef LAUNCH_PREP
 #undef ARGS
   if (lrs_check_launch("attention_decode")) return 1;
-  if (splits > 1) {
-    launch_attention_merge((bf16*)out, out_stride, part_o, part_ml, tokens, nq, d, splits, s);
+  if (keep_first > 0) {
+    launch_attention_kept((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, token_request,
+                          positions, tokens, nq, nkv, d, page_size, scale, window, keep_first, slots, part_o, part_ml, s);
+    if (lrs_check_launch("attention_kept")) return 1;
+  }
+  if (slots > 1) {
+    launch_attention_merge((bf16*)out, out_stride, part_o, part_ml, tokens, nq, d, slots, s);
     return lrs_check_launch("attention_merge");
   }
   return 0;
@@ -684,7 +764,7 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_request,
     const int* __restrict__ positions, const int* __restrict__ qblock_token0,
     const int* __restrict__ qblock_count, int n_blocks, int chunk, int nq, int nkv, int page_size, float scale,
-    int window, int splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    int window, int splits, int slots, float* __restrict__ part_o, float* __restrict__ part_ml) {
   constexpr int DS = D / 32, DB = D / 16;
   // Padded LDS rows.  Every fragment is read 16 bytes a lane, 16 rows at a time (the lane's row is col, its
   // piece g), which the LDS serves at its full 256 bytes a cycle when rows lie 32 bytes more than a multiple
@@ -960,8 +1040,8 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
       float total = run_sum[b];
       total += __shfl_xor(total, 16, WAVE);
       total += __shfl_xor(total, 32, WAVE);
-      if (live[b] && splits > 1) {
-        const int64_t slot = ((int64_t)(token0 + b * 16 + col) * nq + head) * splits + split;
+      if (live[b] && slots > 1) {
+        const int64_t slot = ((int64_t)(token0 + b * 16 + col) * nq + head) * slots + split;
 #pragma unroll
         for (int e = 0; e < DB; ++e) *(floatx4*)(part_o + slot * D + e * 16 + g * 4) = o[b][e];
         if (g == 0) {
@@ -1010,7 +1090,7 @@ __global__ __launch_bounds__(MANY_WAVES ? 512 : 256, MANY_WAVES ? 1 : 2) void at
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_request,
     const int* __restrict__ positions, const int* __restrict__ qblock_token0,
     const int* __restrict__ qblock_count, int n_blocks, int chunk, int nq, int nkv, int page_size, float scale,
-    int window, int splits, float* __restrict__ part_o, float* __restrict__ part_ml, int prepare_q, DecodePrep prep) {
+    int window, int splits, int slots, float* __restrict__ part_o, float* __restrict__ part_ml, int prepare_q, DecodePrep prep) {
   constexpr int D = 128, DS = D / 32, DB = D / 16, STAGES = 3;
   constexpr int KBLOCK = 1024 + 32, KBYTES = 8 * KBLOCK, VHALF = 16 * D * 2 + 16, VBYTES = 2 * VHALF;
   constexpr int VSTAGE = (VBYTES + 63) / 64 * 64;
@@ -1361,8 +1441,8 @@ __global__ __launch_bounds__(MANY_WAVES ? 512 : 256, MANY_WAVES ? 1 : 2) void at
       float total = run_sum[b];
       total += __shfl_xor(total, 16, WAVE);
       total += __shfl_xor(total, 32, WAVE);
-      if (live[b] && splits > 1) {
-        const int64_t slot = ((int64_t)(token0 + b * 16 + col) * nq + head) * splits + split;
+      if (live[b] && slots > 1) {
+        const int64_t slot = ((int64_t)(token0 + b * 16 + col) * nq + head) * slots + split;
 #pragma unroll
         for (int e = 0; e < DB; ++e) *(floatx4*)(part_o + slot * D + e * 16 + g * 4) = o[b][e];
         if (g == 0) {
@@ -1426,7 +1506,7 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
                                   const void* v_pages, const int* block_table, int table_stride,
                                   const int* token_request, const int* positions, const int* qblock_token0,
                                   const int* qblock_count, int n_blocks, int max_count, int max_context, int nq,
-                                  int nkv, int d, int page_size, float scale, int window, int tokens, int splits,
+                                  int nkv, int d, int page_size, float scale, int window, int keep_first, int tokens, int splits,
                                   float* part_o, float* part_ml, int prepare, const void* q_weight, int w_dtype, float eps,
                                   const float* cosv, const float* sinv, void* stream) {
   LRS_REQUIRE(n_blocks > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_prefill: bad sizes blocks=%d nq=%d nkv=%d", n_blocks, nq, nkv);
@@ -1440,13 +1520,15 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
   const DecodePrep prep{q_weight, nullptr, w_dtype == LRS_F32, eps, cosv, sinv, 0};
   LRS_REQUIRE(max_count >= 1 && max_count <= 32, "attention_prefill: query groups hold 1..32 tokens, got %d", max_count);
   LRS_REQUIRE(page_size % 16 == 0, "attention_prefill: page size %d is not a multiple of 16", page_size);
-  LRS_REQUIRE(window >= 0, "attention_prefill: window must be >= 0 (0 = none)");
+  LRS_REQUIRE(window >= 0 && keep_first >= 0 && (keep_first == 0 || (window > 0 && !prepare)),
+              "attention_prefill: kept first positions (%d) need a window and prepared heads", keep_first);
+  const int slots = splits + (keep_first > 0 ? 1 : 0);          // the kept keys' share is one more partial result
   LRS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && out_stride % 4 == 0 && ((uintptr_t)out % 8) == 0,
               "attention_prefill: q rows must be 16-byte and out rows 8-byte aligned");
   // four waves (with fewer heads in a kv group the spare waves still help to bring tiles in), more only below
-  LRS_REQUIRE(splits >= 1 && splits <= 64 && (splits == 1 || (part_o && part_ml && tokens > 0)),
+  LRS_REQUIRE(splits >= 1 && splits <= 64 && (slots == 1 || (part_o && part_ml && tokens > 0)),
               "attention_prefill: splits=%d (1..64) need partial buffers and the number of tokens", splits);
-  LRS_REQUIRE(splits == 1 || ((uintptr_t)part_o % 16) == 0, "attention_prefill: part_o must be 16-byte aligned");
+  LRS_REQUIRE(slots == 1 || ((uintptr_t)part_o % 16) == 0, "attention_prefill: part_o must be 16-byte aligned");
   dim3 grid(n_blocks * nkv * splits), block(4 * WAVE);
   // workgroups that share a compute unit: see the kernel
   const int chunk = nkv >= compute_units() ? nkv : compute_units() / nkv * nkv;
@@ -1462,7 +1544,7 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
                                                               (const bf16*)k_pages, (const bf16*)v_pages, block_table, \
                                                               table_stride, token_request, positions, qblock_token0, \
                                                               qblock_count, n_blocks, chunk, nq, nkv, page_size, scale, window, \
-                                                              splits, part_o, part_ml)
+                                                              splits, slots, part_o, part_ml)
 #define LAUNCH(D)                                \
   if (max_count <= 16) LAUNCH2(D, 1);            \
   else LAUNCH2(D, 2)
@@ -1481,7 +1563,7 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
 #define D128(QB, MANY, IDLE)                                                                                                      \
         attention_prefill_d128_bf16_kernel<QB, MANY, IDLE><<<grid, block, 0, s>>>(                                                    \
             (bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, \
-            token_request, positions, qblock_token0, qblock_count, n_blocks, chunk, nq, nkv, page_size, scale, window, splits, part_o, part_ml, \
+            token_request, positions, qblock_token0, qblock_count, n_blocks, chunk, nq, nkv, page_size, scale, window, splits, slots, part_o, part_ml, \
             prepare, prep)
 #define D128_OF(QB)                                      \
         if (many && idle) D128(QB, true, true);          \
@@ -1501,8 +1583,13 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
 #undef LAUNCH
 #undef LAUNCH2
   if (lrs_check_launch("attention_prefill")) return 1;
-  if (splits > 1) {
-    launch_attention_merge((bf16*)out, out_stride, part_o, part_ml, tokens, nq, d, splits, s);
+  if (keep_first > 0) {
+    launch_attention_kept((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, token_request,
+                          positions, tokens, nq, nkv, d, page_size, scale, window, keep_first, slots, part_o, part_ml, s);
+    if (lrs_check_launch("attention_kept")) return 1;
+  }
+  if (slots > 1) {
+    launch_attention_merge((bf16*)out, out_stride, part_o, part_ml, tokens, nq, d, slots, s);
     return lrs_check_launch("attention_merge");
   }
   return 0;

@@ -131,7 +131,8 @@ def random_model(config, seed: int, dtype: torch.dtype, device, init: str = "nor
     model = DecoderModel(spec)
     # drawn in the precision the architecture's checkpoints are stored in, and brought to the device as a loaded
     # checkpoint is: float16, which no kernel takes, widened to float32
-    drawn = device_weights(model, seed, TORCH_DTYPES[spec.checkpoint_dtype], device, init)
+    # sizes that a part reads from its checkpoint (a low-rank input's rank) are what the configuration says random weights take
+    drawn = device_weights(model, seed, TORCH_DTYPES[spec.checkpoint_dtype], device, init, free_size=getattr(config, "random_rank", None))
 
     def widened(name: str) -> torch.Tensor:
         t = drawn[name]

@@ -137,10 +137,10 @@ _SIGNATURES = {
                         c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_float,
                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "lrs_attention_decode": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
-                                     c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int,
+                                     c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int,
                                      c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_attention_prefill": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
-                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
+                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
                                       c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p]),
     "lrs_attention_prefill_prepares": (c_int, [c_int]),
     "lrs_compute_units": (c_int, []),
@@ -1070,9 +1070,11 @@ def decode_prepare_supported(d: int, rotates: bool) -> bool:
 def attention_decode(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                      token_request: torch.Tensor, positions: torch.Tensor, nq: int, scale: float, window: int = 0, splits: int = 1,
                      part_o: torch.Tensor | None = None, part_ml: torch.Tensor | None = None, max_context: int | None = None,
-                     prepare: "DecodePrepare | None" = None, form: int = 0) -> None:
+                     prepare: "DecodePrepare | None" = None, form: int = 0, keep_first: int = 0) -> None:
     """attention() for a step with one query token per request, bfloat16 only; the keys of a token
     are divided between `splits` workgroups whose partial results meet in part_o / part_ml.
+    keep_first (with a window and prepared heads): the first positions of a sequence stay visible behind the window; their
+    share is one more partial result, so the buffers hold splits + 1 and are needed whatever `splits` is.
 
     prepare: `q` holds the raw rows of the q/k/v product and the kernel also does what qk_prep()
     does (see DecodePrepare); without it q, and the pages, must have been through qk_prep()."""
@@ -1086,9 +1088,11 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, 
     _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.stride(1) == 1, "attention_decode: block_table must be int32 [R, blocks]")
     for name, t in (("token_request", token_request), ("positions", positions)):
         _need(t.dtype == torch.int32 and t.numel() >= tokens and t.is_contiguous(), f"attention_decode: {name} must be int32 [T]")
-    if splits > 1:
-        _need(part_o is not None and part_o.dtype == torch.float32 and part_o.is_contiguous() and part_o.numel() >= tokens * nq * splits * d, "attention_decode: part_o too small")
-        _need(part_ml is not None and part_ml.dtype == torch.float32 and part_ml.is_contiguous() and part_ml.numel() >= tokens * nq * splits * 2, "attention_decode: part_ml too small")
+    _need(keep_first >= 0 and (keep_first == 0 or (window > 0 and prepare is None)), "attention_decode: kept first positions need a window and prepared heads")
+    slots = splits + (1 if keep_first else 0)
+    if slots > 1:
+        _need(part_o is not None and part_o.dtype == torch.float32 and part_o.is_contiguous() and part_o.numel() >= tokens * nq * slots * d, "attention_decode: part_o too small")
+        _need(part_ml is not None and part_ml.dtype == torch.float32 and part_ml.is_contiguous() and part_ml.numel() >= tokens * nq * slots * 2, "attention_decode: part_ml too small")
     fused = [0, None, None, 0, 0.0, None, None, 0]
     if prepare is not None:
         _need(decode_prepare_supported(d, prepare.cos is not None), f"attention_decode: cannot rotate heads of {d} dims itself")
@@ -1105,10 +1109,10 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, 
                  dtype_code(prepare.q_weight.dtype) if normed else 0, prepare.eps,
                  None if prepare.cos is None else _dev(prepare.cos, "cos"), None if prepare.sin is None else _dev(prepare.sin, "sin"), prepare.kv_heads]
     _launch("lrs_attention_decode", 
-        _dev(out, "out"), _rows(out, "out"), None if splits == 1 else _dev(part_o, "part_o"), None if splits == 1 else _dev(part_ml, "part_ml"),
+        _dev(out, "out"), _rows(out, "out"), None if slots == 1 else _dev(part_o, "part_o"), None if slots == 1 else _dev(part_ml, "part_ml"),
         _dev(q, "q"), _rows(q, "q"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(block_table, "block_table"), block_table.stride(0),
         _dev(token_request, "token_request"), _dev(positions, "positions"), tokens,
-        block_table.shape[1] * page_size if max_context is None else max_context, nq, nkv, d, page_size, scale, window, splits,
+        block_table.shape[1] * page_size if max_context is None else max_context, nq, nkv, d, page_size, scale, window, keep_first, splits,
         form, *fused, _stream())
 
 
@@ -1116,7 +1120,7 @@ def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor,
                       token_request: torch.Tensor, positions: torch.Tensor, qblock_token0: torch.Tensor, qblock_count: torch.Tensor,
                       nq: int, scale: float, window: int = 0, max_count: int | None = None, max_context: int | None = None,
                       splits: int = 1, part_o: torch.Tensor | None = None, part_ml: torch.Tensor | None = None,
-                      prepare: "DecodePrepare | None" = None) -> None:
+                      prepare: "DecodePrepare | None" = None, keep_first: int = 0) -> None:
     """attention() on matrix cores for any bfloat16 step.  qblock_token0 / qblock_count list groups of at
     most attention_prefill_group() consecutive tokens of one request that together cover every token of
     the step once; `max_count` is the largest count among them (the group limit if not given) and
@@ -1125,7 +1129,9 @@ def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor,
     their partial results meet in part_o [T, nq * splits * d] and part_ml [T, nq * splits * 2] float32.
     prepare (where attention_prefill_prepares(d)): `q` holds the raw q heads of the q/k/v product, and the kernel gives
     them their norm and rotation itself (q_weight, eps, cos, sin of DecodePrepare; kv_heads 0: the keys and values are in
-    the pages already, from qk_prep(skip_q=True))."""
+    the pages already, from qk_prep(skip_q=True)).
+    keep_first (with a window and prepared heads): the first positions of a sequence stay visible behind the window; their
+    share is one more partial result, so the buffers hold splits + 1 and are needed whatever `splits` is."""
     tokens = out.shape[0]
     _need(k_pages.dim() == 4 and k_pages.is_contiguous() and v_pages.is_contiguous(), "attention_prefill: pages must be contiguous")
     _, nkv, page_size, d = k_pages.shape
@@ -1140,9 +1146,11 @@ def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor,
     _need(n_blocks > 0 and qblock_count.numel() == n_blocks and qblock_token0.dtype == qblock_count.dtype == torch.int32
           and qblock_token0.is_contiguous() and qblock_count.is_contiguous(), "attention_prefill: query blocks must be two int32 vectors of one length")
     _need(1 <= splits <= 64, f"attention_prefill: splits must be 1..64, got {splits}")
-    if splits > 1:
-        _need(part_o is not None and part_o.dtype == torch.float32 and part_o.is_contiguous() and part_o.numel() >= tokens * nq * splits * d, "attention_prefill: part_o too small")
-        _need(part_ml is not None and part_ml.dtype == torch.float32 and part_ml.is_contiguous() and part_ml.numel() >= tokens * nq * splits * 2, "attention_prefill: part_ml too small")
+    _need(keep_first >= 0 and (keep_first == 0 or (window > 0 and prepare is None)), "attention_prefill: kept first positions need a window and prepared heads")
+    slots = splits + (1 if keep_first else 0)
+    if slots > 1:
+        _need(part_o is not None and part_o.dtype == torch.float32 and part_o.is_contiguous() and part_o.numel() >= tokens * nq * slots * d, "attention_prefill: part_o too small")
+        _need(part_ml is not None and part_ml.dtype == torch.float32 and part_ml.is_contiguous() and part_ml.numel() >= tokens * nq * slots * 2, "attention_prefill: part_ml too small")
     fused = [0, None, 0, 0.0, None, None]
     if prepare is not None:
         _need(attention_prefill_prepares(d), f"attention_prefill: heads of {d} dims must come prepared")
@@ -1160,8 +1168,8 @@ def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor,
         _dev(block_table, "block_table"), block_table.stride(0), _dev(token_request, "token_request"), _dev(positions, "positions"),
         _dev(qblock_token0, "qblock_token0"), _dev(qblock_count, "qblock_count"), n_blocks,
         attention_prefill_group() if max_count is None else max_count,
-        block_table.shape[1] * page_size if max_context is None else max_context, nq, nkv, d, page_size, scale, window,
-        tokens, splits, None if splits == 1 else _dev(part_o, "part_o"), None if splits == 1 else _dev(part_ml, "part_ml"), *fused, _stream())
+        block_table.shape[1] * page_size if max_context is None else max_context, nq, nkv, d, page_size, scale, window, keep_first,
+        tokens, splits, None if slots == 1 else _dev(part_o, "part_o"), None if slots == 1 else _dev(part_ml, "part_ml"), *fused, _stream())
 
 
 def attention_prefill_prepares(d: int) -> bool:

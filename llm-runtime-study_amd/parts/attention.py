@@ -20,7 +20,8 @@ at once, a weight per column) instead of per head; `value_dim` gives the values 
 first positions of a sequence visible behind a window (token i sees j <= i with i - j < window or j < keep_first; the kept
 keys keep their positions); `output_gate` multiplies the heads' outputs by sigmoid(W_g x) before the output projection (the
 gate's matrix is stacked behind q, k and v).  A layer with any of them prepares its heads with `qkv_norm_prep`; its attention
-runs on the matrix cores where the shape allows (values as wide as keys, no kept positions) and in the any-shape kernel otherwise.
+runs on the matrix cores where the shape allows (bfloat16, values as wide as keys; the kept positions' keys are then one more
+partial result beside those of the window's splits, which the merge of the splits adds in) and in the any-shape kernel otherwise.
 """
 
 from __future__ import annotations
@@ -300,40 +301,43 @@ class GQAAttention(Part):
         ops.qkv_norm_prep(qkv, nq, nkv, d, dv, self.q_norm, self.k_norm, self.qk_norm_eps, cos, sin, cache.k_pages, cache.v_pages,
                           group.slots, group.page_size)
         out = ctx.scratch("attn_out", (t, nq * dv), ctx.dtype)
-        cores = dv == d and not self.keep_first and ops.attention_decode_supported(ctx.dtype, nq, nkv, d, group.page_size)
+        cores = dv == d and ops.attention_decode_supported(ctx.dtype, nq, nkv, d, group.page_size)
+        extra = 1 if self.keep_first else 0      # the kept first positions' share is one more partial result for the merge
         if cores and ctx.all_decode:
             longest, bound = ctx.max_k, ctx.max_k_bound
             if self.window is not None:
                 longest, bound = min(longest, self.window + 32), min(bound, self.window + 64)
             splits = self._decode_splits(t * nkv, longest, bound, group.page_size)
             part_o = part_ml = None
-            if splits > 1:
-                part_o = ctx.scratch("attn_part_o", (t, nq * splits * d), torch.float32)
-                part_ml = ctx.scratch("attn_part_ml", (t, nq * splits * 2), torch.float32)
+            if splits + extra > 1:
+                part_o = ctx.scratch("attn_part_o", (t, nq * (splits + extra) * d), torch.float32)
+                part_ml = ctx.scratch("attn_part_ml", (t, nq * (splits + extra) * 2), torch.float32)
             ops.attention_decode(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_slot, ctx.positions,
-                                 nq, self.scale, self.window or 0, splits, part_o, part_ml, ctx.max_k_bound, None, form=1)
+                                 nq, self.scale, self.window or 0, splits, part_o, part_ml, ctx.max_k_bound, None, form=1,
+                                 keep_first=self.keep_first)
         elif cores:
             longest = ctx.max_k_bound if self.window is None else min(ctx.max_k_bound, self.window + 64)
             singles = ctx.single_rows
             if singles:
                 splits = self._decode_splits(singles * nkv, longest, ctx.max_k_bound, group.page_size)
                 part_o = part_ml = None
-                if splits > 1:
-                    part_o = ctx.scratch("attn_single_part_o", (singles, nq * splits * d), torch.float32)
-                    part_ml = ctx.scratch("attn_single_part_ml", (singles, nq * splits * 2), torch.float32)
+                if splits + extra > 1:
+                    part_o = ctx.scratch("attn_single_part_o", (singles, nq * (splits + extra) * d), torch.float32)
+                    part_ml = ctx.scratch("attn_single_part_ml", (singles, nq * (splits + extra) * 2), torch.float32)
                 ops.attention_decode(out[:singles], qkv[:singles], cache.k_pages, cache.v_pages, group.block_table, ctx.token_slot,
-                                     ctx.positions, nq, self.scale, self.window or 0, splits, part_o, part_ml, ctx.max_k_bound, None, form=1)
+                                     ctx.positions, nq, self.scale, self.window or 0, splits, part_o, part_ml, ctx.max_k_bound, None, form=1,
+                                     keep_first=self.keep_first)
             rest = ctx.memo.get("rows_after_singles")
             if rest is None:
                 rest = ctx.memo["rows_after_singles"] = (ctx.token_slot[singles:], ctx.positions[singles:])
             splits = self._prefill_splits(ctx.num_qblocks * nkv, longest, (t - singles) * nq * d, nq // nkv, t - singles)
             part_o = part_ml = None
-            if splits > 1:
-                part_o = ctx.scratch("attn_part_o", (t - singles, nq * splits * d), torch.float32)
-                part_ml = ctx.scratch("attn_part_ml", (t - singles, nq * splits * 2), torch.float32)
+            if splits + extra > 1:
+                part_o = ctx.scratch("attn_part_o", (t - singles, nq * (splits + extra) * d), torch.float32)
+                part_ml = ctx.scratch("attn_part_ml", (t - singles, nq * (splits + extra) * 2), torch.float32)
             ops.attention_prefill(out[singles:], qkv[singles:], cache.k_pages, cache.v_pages, group.block_table, rest[0], rest[1],
                                   ctx.qblock_token0, ctx.qblock_count, nq, self.scale, self.window or 0, ctx.max_qblock, ctx.max_k_bound,
-                                  splits, part_o, part_ml, None)
+                                  splits, part_o, part_ml, None, keep_first=self.keep_first)
         else:
             ops.attention(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_slot, ctx.positions, nq, self.scale,
                           self.window or 0, self.keep_first)

@@ -851,6 +851,85 @@ def test_attention_decode_kernel(ops, nq, nkv, d, page, window, splits):
     assert torch.equal(results[0], results[1])      # the same sums in the same order
 
 
+@pytest.mark.parametrize("nq,nkv,d,page,window,keep", [(8, 2, 64, 16, 40, 4), (4, 4, 128, 16, 33, 17), (6, 2, 32, 32, 20, 1), (16, 2, 128, 16, 100, 40),
+                                                       (3, 1, 96, 16, 5, 9)])
+def test_attention_behind_a_window_that_keeps_the_first_positions(ops, nq, nkv, d, page, window, keep):
+    """Token p sees j <= p with p - j < window or j < keep.  The kernel for any shape, and the matrix-core kernels for single
+    tokens and for ragged steps, with the window's keys whole and divided between workgroups: the kept keys are one more
+    partial result that the merge adds in.  One kept key is made to outweigh everything inside the window."""
+    g = torch.Generator().manual_seed(26)
+    requests = [(0, 19), (37, 1), (150, 1), (5, 6), (page * 3 - 1, 2), (9, 75), (window + keep - 1, 3), (300, 1)]
+    scale = 1 / math.sqrt(d)
+    max_blocks = max((a + b + page - 1) // page for a, b in requests)
+    n_pages = sum((a + b + page - 1) // page for a, b in requests) + 3
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    kp, vp = torch.randn(n_pages, nkv, page, d, generator=g), torch.randn(n_pages, nkv, d, page, generator=g)
+    table = torch.zeros(len(requests), max_blocks, dtype=torch.int32)
+    rows, tok_req, tok_pos, want = [], [], [], []
+    for r, (before, new) in enumerate(requests):
+        total = before + new
+        k = torch.randn(total, nkv, d, generator=g).bfloat16()
+        v = torch.randn(total, nkv, d, generator=g).bfloat16()
+        q = (torch.randn(new, nq, d, generator=g) * 2).bfloat16()
+        if total > window + keep:
+            k[keep - 1, 0] = (3.0 * q[-1, 0]).bfloat16()          # the last kept key answers the last query's first head loudly
+        for b in range((total + page - 1) // page):
+            pg = perm.pop()
+            table[r, b] = pg
+            n = min(page, total - b * page)
+            kp[pg, :, :n] = k[b * page: b * page + n].float().transpose(0, 1)
+            vp[pg, :, :, :n] = v[b * page: b * page + n].float().permute(1, 2, 0)
+        for i in range(new):
+            p = before + i
+            seen = [j for j in range(p + 1) if p - j < window or j < keep]
+            heads = []
+            for h in range(nq):
+                gi = h // (nq // nkv)
+                weights = torch.softmax((k[seen, gi].double() @ q[i, h].double()) * scale, 0)
+                heads.append(weights @ v[seen, gi].double())
+                if i == new - 1 and h == 0 and total > window + keep:
+                    assert weights[seen.index(keep - 1)] > 0.9
+            want.append(torch.cat(heads))
+            rows.append(q[i])
+            tok_req.append(r)
+            tok_pos.append(p)
+    want, q, t = torch.stack(want), torch.stack(rows), len(rows)
+    q_wide = torch.zeros(t, nq * d + 2 * nkv * d, dtype=torch.bfloat16)
+    q_wide[:, : nq * d] = q.view(t, nq * d)
+    tok_req, tok_pos = torch.tensor(tok_req, dtype=torch.int32), torch.tensor(tok_pos, dtype=torch.int32)
+    for dtype in DTYPES:
+        out = torch.empty(t, nq * d, device="cuda", dtype=dtype)
+        ops.attention(out, dev(q_wide.to(dtype)), dev(kp.bfloat16().to(dtype)), dev(vp.bfloat16().to(dtype)), dev(table), dev(tok_req), dev(tok_pos),
+                      nq, scale, window, keep)
+        torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 2e-5, 2e-2))
+    assert ops.attention_decode_supported(torch.bfloat16, nq, nkv, d, page)
+    pages = (dev(kp.bfloat16()), dev(vp.bfloat16()))
+    for size, splits in ((16, 1), (32, 1), (7, 2), (16, 4), (32, 8)):
+        blocks, at = [], 0
+        for before, new in requests:
+            blocks += [(at + i, min(size, new - i)) for i in range(0, new, size)]
+            at += new
+        fast = torch.full((t, nq * d), float("nan"), device="cuda", dtype=torch.bfloat16)
+        part_o = torch.full((t, nq * (splits + 1) * d), float("nan"), device="cuda")
+        part_ml = torch.full((t, nq * (splits + 1) * 2), float("nan"), device="cuda")
+        ops.attention_prefill(fast, dev(q_wide), *pages, dev(table), dev(tok_req), dev(tok_pos), dev(torch.tensor([b[0] for b in blocks], dtype=torch.int32)),
+                              dev(torch.tensor([b[1] for b in blocks], dtype=torch.int32)), nq, scale, window, size, splits=splits,
+                              part_o=part_o, part_ml=part_ml, keep_first=keep)
+        torch.testing.assert_close(fast.cpu().double(), want, rtol=2e-2, atol=2e-2)
+    # single tokens: the last token of every request, as a step of its own
+    last = [i for i in range(t) if i == t - 1 or tok_req[i + 1] != tok_req[i]]
+    for splits in (1, 3):
+        for form in (0, 1, 2):
+            fast = torch.full((len(last), nq * d), float("nan"), device="cuda", dtype=torch.bfloat16)
+            part_o = torch.full((len(last), nq * (splits + 1) * d), float("nan"), device="cuda")
+            part_ml = torch.full((len(last), nq * (splits + 1) * 2), float("nan"), device="cuda")
+            ops.attention_decode(fast, dev(q_wide[last]), *pages, dev(table), dev(tok_req[last]), dev(tok_pos[last]), nq, scale, window, splits,
+                                 part_o, part_ml, form=form, keep_first=keep)
+            torch.testing.assert_close(fast.cpu().double(), want[last], rtol=2e-2, atol=2e-2)
+    with pytest.raises(Exception, match="kept first positions"):
+        ops.attention_decode(fast, dev(q_wide[last]), *pages, dev(table), dev(tok_req[last]), dev(tok_pos[last]), nq, scale, 0, 1, part_o, part_ml, keep_first=keep)
+
+
 @pytest.mark.parametrize("nq,nkv,d,page,window,splits,normed,rotated,shared", [
     (32, 8, 128, 16, 0, 5, True, True, False), (4, 4, 64, 32, 0, 3, True, True, False), (6, 2, 192, 64, 0, 4, False, True, False),
     (8, 2, 32, 16, 0, 2, True, False, False), (16, 1, 96, 16, 40, 1, False, False, False), (8, 2, 64, 16, 100, 3, True, True, True),
