@@ -40,7 +40,8 @@ __global__ void delta_prepare_kernel(const TP* __restrict__ proj, int ld, const 
                                      int decay_rank, const float* __restrict__ decay_up, float* __restrict__ decays) {
   // beta_at, decay_at: the columns of proj that hold the step sizes (H) and the decay inputs: H of them, or, with
   // decay_rank > 0, decay_rank values that decay_up [decay_rank, H * d] carries to one input per head and key channel
-  // (dt_bias then holds H * d values and decays [tokens, H * d] receives the decays; gates' second half is left alone)
+  // (dt_bias then holds H * d values and decays [tokens, H * d] receives the decays; gates' second half is left alone);
+  // decay_rank < 0: decays holds those H * d inputs of every token already (a product made them) and is turned into the decays in place
   // keep_inside: every request brings one token, so this wave alone reads and writes its channels' kept inputs of its
   // request: it moves them on itself (no delta_conv_keep launch)
   const int t = blockIdx.x, unit = blockIdx.y, lane = threadIdx.x;
@@ -73,10 +74,11 @@ __global__ void delta_prepare_kernel(const TP* __restrict__ proj, int ld, const 
     const int h = unit - 2 * G;
     const int64_t row = (int64_t)t * ld;
     if (lane == 0) gates[(int64_t)t * 2 * H + h] = 1.f / (1.f + expf(-to_float(proj[row + beta_at + h])));
-    if (decay_rank > 0) {
+    if (decay_rank != 0) {
       const float rate = expf(a_log[h]);
       for (int i = lane; i < d; i += WAVE) {
         float a = dt_bias[h * d + i];
+        if (decay_rank < 0) a += decays[(int64_t)t * H * d + h * d + i];
         for (int r = 0; r < decay_rank; ++r) a = fmaf(to_float(proj[row + decay_at + r]), decay_up[(int64_t)r * H * d + h * d + i], a);
         const float softplus = a > 20.f ? a : log1pf(expf(a));
         decays[(int64_t)t * H * d + h * d + i] = expf(-rate * softplus);
@@ -323,7 +325,7 @@ __global__ __launch_bounds__(256) void delta_scan_single_kernel(const float* __r
 
 // The head's read-out divided by its root mean square over vdim, times the norm's weight, times silu(gate): a wave a
 // (token, head).  gate_rank > 0: the gate is sigmoid instead, of the gate_rank values at gate_at carried to H * dv
-// inputs by gate_up [gate_rank, H * dv].
+// inputs by gate_up [gate_rank, H * dv]; gate_rank < 0: gate_up holds those H * dv inputs of every token already, [tokens, H * dv].
 template <typename TP, typename TO>
 __global__ __launch_bounds__(256) void delta_gate_kernel(const float* __restrict__ raw_out, const TP* __restrict__ proj, int ld,
                                                          int gate_at, const float* __restrict__ norm_w, float eps, int tokens, int H,
@@ -340,7 +342,9 @@ __global__ __launch_bounds__(256) void delta_gate_kernel(const float* __restrict
   const float inv = 1.0f / sqrtf(ss / (float)dv + eps);
   for (int i = lane; i < dv; i += WAVE) {
     float factor;
-    if (gate_rank > 0) {
+    if (gate_rank < 0) {
+      factor = 1.f / (1.f + expf(-gate_up[token * H * dv + (int64_t)h * dv + i]));
+    } else if (gate_rank > 0) {
       float gate = 0.f;
       for (int r = 0; r < gate_rank; ++r) gate = fmaf(to_float(proj[token * ld + gate_at + r]), gate_up[(int64_t)r * H * dv + h * dv + i], gate);
       factor = 1.f / (1.f + expf(-gate));
@@ -451,7 +455,8 @@ namespace {
 
 // The gated delta rule's kernels for one step.  gate_at, beta_at, decay_at: columns of proj.  decay_rank > 0: a decay per
 // head and key channel from decay_rank values (decay_up [decay_rank, H*d], dt_bias [H*d], decays [tokens, H*d] scratch);
-// gate_rank > 0: a sigmoid gate from gate_rank values (gate_up [gate_rank, H*dv]); else silu of H*dv columns.
+// gate_rank > 0: a sigmoid gate from gate_rank values (gate_up [gate_rank, H*dv]); 0: silu of H*dv columns.  A rank below 0:
+// the inputs were made by a product of the caller's: decays [tokens, H*d] holds the decays' inputs, gate_up [tokens, H*dv] the gate's.
 int delta_launch(void* out, int out_dtype, const void* proj, int proj_dtype, int ld, int tokens, int requests,
                  const int* token_request, const int* cu, const int* slot_ids, float* state, int64_t state_stride,
                  const float* conv_w, int taps, int G, int H, int d, int dv, const float* a_log, const float* dt_bias,
@@ -461,15 +466,16 @@ int delta_launch(void* out, int out_dtype, const void* proj, int proj_dtype, int
   LRS_REQUIRE(G > 0 && H > 0 && H % G == 0 && d > 0 && dv > 0 && taps >= 1, "delta_rule: bad sizes G=%d H=%d d=%d dv=%d taps=%d", G, H, d, dv, taps);
   LRS_REQUIRE(d <= 256, "delta_rule: takes keys of up to 256 values, got %d", d);
   const int rows = lrs_delta_state_rows(d), channels = 2 * G * d + H * dv;
-  const int last = gate_at + (gate_rank > 0 ? gate_rank : H * dv) > decay_at + (decay_rank > 0 ? decay_rank : H)
-                       ? gate_at + (gate_rank > 0 ? gate_rank : H * dv) : decay_at + (decay_rank > 0 ? decay_rank : H);
+  const int gate_end = gate_rank < 0 ? 0 : gate_at + (gate_rank > 0 ? gate_rank : H * dv);
+  const int decay_end = decay_rank < 0 ? 0 : decay_at + (decay_rank > 0 ? decay_rank : H);
+  const int last = gate_end > decay_end ? gate_end : decay_end;
   LRS_REQUIRE(ld >= channels && ld >= last && ld >= beta_at + H, "delta_rule: projection rows of %d hold fewer than the columns needed", ld);
   const int64_t conv_offset = (int64_t)H * rows * SPLIT * dv;
   LRS_REQUIRE(state_stride >= conv_offset + (int64_t)(taps - 1) * channels, "delta_rule: a state row of %lld floats is too short", (long long)state_stride);
   LRS_REQUIRE(eps > 0.f, "delta_rule: eps must be positive");
   LRS_REQUIRE(((uintptr_t)qkv % 16) == 0 && ((uintptr_t)decays % 16) == 0, "delta_rule: the scratch rows must be 16 bytes aligned");
-  LRS_REQUIRE(decay_rank == 0 || (decay_up && decays), "delta_rule: decays per channel need their matrix and scratch rows");
-  LRS_REQUIRE(gate_rank == 0 || gate_up, "delta_rule: a gate of low rank needs its matrix");
+  LRS_REQUIRE(decay_rank == 0 || ((decay_up || decay_rank < 0) && decays), "delta_rule: decays per channel need their matrix and scratch rows");
+  LRS_REQUIRE(gate_rank == 0 || gate_up, "delta_rule: a gate of low rank needs its matrix or its inputs");
   hipStream_t s = (hipStream_t)stream;
   dim3 pgrid(tokens, 2 * G + H), kgrid(requests, (channels + 255) / 256), sgrid(requests, H, (dv + COLUMNS - 1) / COLUMNS);
   const int64_t pairs = (int64_t)tokens * H;
@@ -482,7 +488,7 @@ int delta_launch(void* out, int out_dtype, const void* proj, int proj_dtype, int
     if (taps > 1 && !single)                                                                                                  \
       delta_conv_keep_kernel<TP><<<kgrid, 256, 0, s>>>((const TP*)proj, ld, cu, slot_ids, state, state_stride, conv_offset,  \
                                                        taps, channels, 0);                                                    \
-    if (decay_rank > 0) launch_scan<RULE_DELTA_CHANNELS>(rows, single, sgrid, s, qkv, gates, cu, slot_ids, state, state_stride, G, H, d, dv, raw, decays); \
+    if (decay_rank != 0) launch_scan<RULE_DELTA_CHANNELS>(rows, single, sgrid, s, qkv, gates, cu, slot_ids, state, state_stride, G, H, d, dv, raw, decays); \
     else launch_scan<RULE_DELTA>(rows, single, sgrid, s, qkv, gates, cu, slot_ids, state, state_stride, G, H, d, dv, raw, nullptr);                    \
     delta_gate_kernel<TP, TO><<<(unsigned)((pairs + 3) / 4), 256, 0, s>>>(raw, (const TP*)proj, ld, gate_at, norm_w, eps, tokens, H, dv, (TO*)out, \
                                                                           gate_rank, gate_up);                                \
@@ -511,13 +517,15 @@ LRS_API int lrs_delta_rule(void* out, int out_dtype, const void* proj, int proj_
 
 // The rule with a decay per head and key channel and a sigmoid gate, both from inputs of low rank.  proj columns:
 // q (G*d) | k (G*d) | v (H*dv) | step size (H) | decay input (decay_rank) | gate input (gate_rank); decay_up [decay_rank, H*d],
-// dt_bias [H*d], gate_up [gate_rank, H*dv], decays [tokens, H*d] float32 scratch.
+// dt_bias [H*d], gate_up [gate_rank, H*dv], decays [tokens, H*d] float32 scratch.  Both ranks -1: the caller has applied the
+// second matrices itself; proj ends with the step sizes, decays holds W_a2 (W_a1 x) and gate_up W_g2 (W_g1 x), [tokens, H*d] and [tokens, H*dv].
 LRS_API int lrs_delta_rule_channels(void* out, int out_dtype, const void* proj, int proj_dtype, int ld, int tokens, int requests,
                                     const int* token_request, const int* cu, const int* slot_ids, float* state, int64_t state_stride,
                                     const float* conv_w, int taps, int G, int H, int d, int dv, const float* a_log,
                                     const float* dt_bias, const float* norm_w, float eps, float* qkv, float* gates, float* raw,
                                     int decay_rank, const float* decay_up, float* decays, int gate_rank, const float* gate_up, void* stream) {
-  LRS_REQUIRE(decay_rank > 0 && gate_rank > 0, "delta_rule_channels: ranks must be positive, got %d and %d", decay_rank, gate_rank);
+  LRS_REQUIRE((decay_rank > 0 && gate_rank > 0) || (decay_rank == -1 && gate_rank == -1),
+              "delta_rule_channels: ranks must both be positive, or both -1 for inputs that are given, got %d and %d", decay_rank, gate_rank);
   const int channels = 2 * G * d + H * dv;
   return delta_launch(out, out_dtype, proj, proj_dtype, ld, tokens, requests, token_request, cu, slot_ids, state, state_stride, conv_w, taps,
                       G, H, d, dv, a_log, dt_bias, norm_w, eps, qkv, gates, raw, channels + H + decay_rank, channels, channels + H, decay_rank,

@@ -1299,23 +1299,34 @@ def delta_rule(out: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, token
 def delta_rule_channels(out: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, token_request: torch.Tensor, cu_seqlens: torch.Tensor,
                         slot_ids: torch.Tensor, requests: int, conv_weight: torch.Tensor, kv_heads: int, heads: int, dim: int, vdim: int,
                         a_log: torch.Tensor, dt_bias: torch.Tensor, norm_weight: torch.Tensor, eps: float, qkv: torch.Tensor, gates: torch.Tensor,
-                        raw: torch.Tensor, decay_up: torch.Tensor, decays: torch.Tensor, gate_up: torch.Tensor) -> None:
+                        raw: torch.Tensor, decay_up: torch.Tensor | None, decays: torch.Tensor, gate_up: torch.Tensor | None,
+                        gate_in: torch.Tensor | None = None) -> None:
     """The gated delta rule with a decay per head and key channel and a sigmoid output gate, both from inputs of low rank.
     proj [T, >= C] columns: q (kv_heads*dim) | k (kv_heads*dim) | v (heads*vdim) | step size (heads) | decay input (rank_a) |
     gate input (rank_g); decay_up float32 [rank_a, heads*dim], dt_bias [heads*dim], gate_up float32 [rank_g, heads*vdim];
-    decays [T, heads*dim] float32 scratch.  Everything else as delta_rule()."""
+    decays [T, heads*dim] float32 scratch.  With decay_up and gate_up None the second matrices have been applied by the
+    caller: `decays` holds the decays' inputs (before bias and softplus) and is turned into the decays in place, `gate_in`
+    [T, heads*vdim] float32 holds the gate's.  Everything else as delta_rule()."""
     tokens = out.shape[0]
     channels = 2 * kv_heads * dim + heads * vdim
     taps = conv_weight.shape[1]
-    rank_a, rank_g = decay_up.shape[0], gate_up.shape[0]
+    given = decay_up is None
+    _need(given == (gate_up is None) and given == (gate_in is not None), "delta_rule_channels: both second matrices, or both of their outputs")
+    rank_a, rank_g = (-1, -1) if given else (decay_up.shape[0], gate_up.shape[0])
     _need(out.is_contiguous() and out.shape[1] == heads * vdim, "delta_rule_channels: out must be contiguous [T, heads*vdim]")
-    _need(proj.shape[0] >= tokens and proj.shape[1] >= channels + heads + rank_a + rank_g, "delta_rule_channels: proj holds too few columns")
+    _need(proj.shape[0] >= tokens and proj.shape[1] >= channels + heads + max(rank_a, 0) + max(rank_g, 0), "delta_rule_channels: proj holds too few columns")
     _need(state.dim() == 2 and state.dtype == torch.float32 and state.is_contiguous()
           and state.shape[1] >= delta_state_floats(heads, kv_heads, dim, vdim, taps), "delta_rule_channels: state rows are too short")
     _need(conv_weight.shape == (channels, taps) and conv_weight.dtype == torch.float32 and conv_weight.is_contiguous(),
           f"delta_rule_channels: the convolution's weights must be float32 [{channels}, taps]")
-    for name, t, shape in (("a_log", a_log, (heads,)), ("dt_bias", dt_bias, (heads * dim,)), ("norm_weight", norm_weight, (vdim,)),
-                           ("decay_up", decay_up, (rank_a, heads * dim)), ("gate_up", gate_up, (rank_g, heads * vdim))):
+    vectors = [("a_log", a_log, (heads,)), ("dt_bias", dt_bias, (heads * dim,)), ("norm_weight", norm_weight, (vdim,))]
+    if given:
+        _need(gate_in.dtype == torch.float32 and gate_in.is_contiguous() and gate_in.dim() == 2 and gate_in.shape[0] >= tokens
+              and gate_in.shape[1] == heads * vdim, f"delta_rule_channels: gate_in must be contiguous float32 [T, {heads * vdim}]")
+        _need(decays.dim() == 2 and decays.shape[1] == heads * dim, f"delta_rule_channels: given decay inputs must be [T, {heads * dim}]")
+    else:
+        vectors += [("decay_up", decay_up, (rank_a, heads * dim)), ("gate_up", gate_up, (rank_g, heads * vdim))]
+    for name, t, shape in vectors:
         _need(t.dtype == torch.float32 and tuple(t.shape) == shape and t.is_contiguous(), f"delta_rule_channels: {name} must be float32 {shape}")
     for name, t, count in (("token_request", token_request, tokens), ("cu_seqlens", cu_seqlens, requests + 1), ("slot_ids", slot_ids, requests)):
         _need(t.dtype == torch.int32 and t.numel() >= count and t.is_contiguous(), f"delta_rule_channels: {name} must be int32 [{count}]")
@@ -1325,8 +1336,8 @@ def delta_rule_channels(out: torch.Tensor, proj: torch.Tensor, state: torch.Tens
     _launch("lrs_delta_rule_channels", _dev(out, "out"), dtype_code(out.dtype), _dev(proj, "proj"), dtype_code(proj.dtype), _rows(proj, "proj"), tokens,
             requests, _dev(token_request, "token_request"), _dev(cu_seqlens, "cu_seqlens"), _dev(slot_ids, "slot_ids"), _dev(state, "state"),
             state.stride(0), _dev(conv_weight, "conv_weight"), taps, kv_heads, heads, dim, vdim, _dev(a_log, "a_log"), _dev(dt_bias, "dt_bias"),
-            _dev(norm_weight, "norm_weight"), eps, _dev(qkv, "qkv"), _dev(gates, "gates"), _dev(raw, "raw"), rank_a, _dev(decay_up, "decay_up"),
-            _dev(decays, "decays"), rank_g, _dev(gate_up, "gate_up"), _stream())
+            _dev(norm_weight, "norm_weight"), eps, _dev(qkv, "qkv"), _dev(gates, "gates"), _dev(raw, "raw"), rank_a,
+            None if given else _dev(decay_up, "decay_up"), _dev(decays, "decays"), rank_g, _dev(gate_in if given else gate_up, "gate_up"), _stream())
 
 
 def state_space(out: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, token_request: torch.Tensor, cu_seqlens: torch.Tensor,

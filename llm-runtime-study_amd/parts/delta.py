@@ -14,8 +14,9 @@ every run; the projections that feed them are written in float32 too.
 `channel_decay` (with `decay_rank`, `gate_rank`): the decay is one number per head and key channel, multiplying the rows of S,
     g = exp(-exp(A_log_h) * softplus(W_a2 (W_a1 x) + dt_bias))  laid out heads x head_dim, dt_bias of that size,
 and the output gate is sigmoid(W_g2 (W_g1 x)) laid out heads x value_dim; W_a1 and W_g1 are stacked behind q, k, v and the step
-size, the second matrices are applied in float32 inside the recurrence's kernels.  A rank of None is read from the checkpoint's
-tensors when they are bound.
+size.  The second matrices are applied in float32: as two products of their own, or, for ranks of at most UPS_IN_KERNEL_RANK (a
+handful of multiply-adds an output cost less than two more launches), inside the recurrence's kernels.  A rank of None is read from
+the checkpoint's tensors when they are bound.
 
 All six input projections are one stacked product.  What a request keeps between steps is one float32 row: the
 matrices of all heads, then the convolution's last taps - 1 inputs of every channel (`StateNeed`); the cache
@@ -39,6 +40,8 @@ def state_rows(head_dim: int) -> int:
 
 
 class GatedDeltaRule(Part):
+    UPS_IN_KERNEL_RANK = 8
+
     graph_safe = True   # launches only this package's kernels on arena buffers, reads the step's data on the device
     plan_safe = True
     can_overwrite = True
@@ -65,7 +68,7 @@ class GatedDeltaRule(Part):
             if value is not None and value <= 0:
                 raise ValueError(f"{name} must be positive when given, got {value}")
         self.channel_decay, self.decay_rank, self.gate_rank = channel_decay, decay_rank, gate_rank
-        self.w_in = self.w_o = self.conv = self.a_log = self.dt_bias = self.norm = self.decay_up = self.gate_up = None
+        self.w_in = self.w_o = self.conv = self.a_log = self.dt_bias = self.norm = self.decay_up = self.gate_up = self.decay_w = self.gate_w = None
 
     def _projections(self):
         qk, v = self.num_kv_heads * self.head_dim, self.num_heads * self.value_dim
@@ -106,9 +109,12 @@ class GatedDeltaRule(Part):
             if (first["a1_proj"], first["g1_proj"]) != (self.decay_up.shape[0], self.gate_up.shape[0]):
                 raise ValueError(f"the two matrices of a low-rank input disagree: {first} against {self.decay_up.shape[0]} and {self.gate_up.shape[0]}")
             self.decay_rank, self.gate_rank = self.decay_up.shape[0], self.gate_up.shape[0]
+            # ... and as stored, [outputs, rank], for the products
+            self.decay_w, self.gate_w = weights["a2_proj.weight"].float().contiguous(), weights["g2_proj.weight"].float().contiguous()
 
     def weight_bytes(self):
-        return (self.w_in.numel() + self.w_o.numel()) * self.w_o.element_size()
+        ups = (self.decay_w.numel() + self.gate_w.numel()) * 4 if self.channel_decay else 0
+        return (self.w_in.numel() + self.w_o.numel()) * self.w_o.element_size() + ups
 
     def flops(self, tokens, pairs):
         # the projections, and per token and head the two products with the state and its update
@@ -133,9 +139,17 @@ class GatedDeltaRule(Part):
         raw = ctx.scratch("delta_read_out", (t, self.num_heads * self.value_dim), torch.float32)
         if self.channel_decay:
             decays = ctx.scratch("delta_decays", (t, self.num_heads * self.head_dim), torch.float32)
+            if max(self.decay_rank, self.gate_rank) <= self.UPS_IN_KERNEL_RANK:
+                decay_up, gate_up, gate_in = self.decay_up, self.gate_up, None
+            else:
+                first = self.channels + self.num_heads
+                gate_in = ctx.scratch("delta_gate_in", (t, self.num_heads * self.value_dim), torch.float32)
+                linear(ctx, decays, proj[:, first:first + self.decay_rank], self.decay_w)
+                linear(ctx, gate_in, proj[:, first + self.decay_rank:first + self.decay_rank + self.gate_rank], self.gate_w)
+                decay_up = gate_up = None
             ops.delta_rule_channels(out, proj, cache.state, ctx.token_request, ctx.cu_seqlens_q, ctx.slot_ids, ctx.R, self.conv, self.num_kv_heads,
                                     self.num_heads, self.head_dim, self.value_dim, self.a_log, self.dt_bias, self.norm, self.norm_eps, qkv, gates, raw,
-                                    self.decay_up, decays, self.gate_up)
+                                    decay_up, decays, gate_up, gate_in)
             linear(ctx, residual, out, self.w_o, accumulate=accumulate)
             return None
         ops.delta_rule(out, proj, cache.state, ctx.token_request, ctx.cu_seqlens_q, ctx.slot_ids, ctx.R, self.conv, self.num_kv_heads,
