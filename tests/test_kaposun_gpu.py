@@ -210,18 +210,21 @@ def test_dense_feed_forward_part(dtype, kind):
     close(out, act @ named["down"].T, dtype, f32=3e-5, bf16=1.5e-2)
 
 
-def test_sum_into_the_stream_leaves_the_next_norm():
+@pytest.mark.parametrize("cols", [136, 135, 4096, 8200])
+def test_sum_into_the_stream_leaves_the_next_norm(cols):
+    """Rows of a multiple of four values up to 8,192 go through the kernel that keeps them in registers, the others through
+    the plain one."""
     from llm_runtime_study_amd.kernels import ops
 
-    h, y = torch.randn(9, 136), 3 * torch.randn(9, 136)
-    weight = (1 + 0.2 * torch.randn(136)).to(torch.bfloat16).float()
+    h, y = torch.randn(9, cols), 3 * torch.randn(9, cols)
+    weight = (1 + 0.2 * torch.randn(cols)).to(torch.bfloat16).float()
     want = h.double() + 0.3 * y.double()
     for dtype in DTYPES:
-        stream, normed = h.clone().cuda(), torch.empty(9, 136, dtype=dtype, device="cuda")
+        stream, normed = h.clone().cuda(), torch.empty(9, cols, dtype=dtype, device="cuda")
         ops.axpby(stream, stream, 1.0, y.cuda(), 0.3, weight.cuda(), 1e-3, normed)
         torch.testing.assert_close(stream.cpu().double(), want, rtol=1e-6, atol=1e-6)
         close(normed, plain.unit_rms(want, 1e-3) * weight.double(), dtype, f32=1e-5, bf16=5e-3)
-    out = torch.empty(9, 136, device="cuda")
+    out = torch.empty(9, cols, device="cuda")
     ops.axpby(out, h.cuda(), 0.8, y.cuda(), 1.5)
     torch.testing.assert_close(out.cpu().double(), 0.8 * h.double() + 1.5 * y.double(), rtol=1e-6, atol=1e-6)
 
