@@ -132,16 +132,22 @@ __global__ __launch_bounds__(256) void qkv_norm_prep_vec_kernel(bf16* __restrict
     const int wbase = (is_q ? head : head - nq) * d;
     const float inv = is_q ? inv_q : inv_k;
     bf16* dst = is_q ? row + (int64_t)head * d : k_pages + ((page * nkv + (head - nq)) * page_size + off) * d;
+    const floatx4 one4 = {1.f, 1.f, 1.f, 1.f};
     if (j < rot8) {
+      // weights and angles of the eight pairs, 16 bytes a load, all asked for before any is used
+      floatx4 wa[2], wb[2], c4[2], s4[2];
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        wa[half] = weight ? *(const floatx4*)(weight + wbase + j * 8 + half * 4) : one4;
+        wb[half] = weight ? *(const floatx4*)(weight + wbase + j * 8 + rot_half + half * 4) : one4;
+        c4[half] = *(const floatx4*)(cosrow + j * 8 + half * 4);
+        s4[half] = *(const floatx4*)(sinrow + j * 8 + half * 4);
+      }
       bf16x8 first, second;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        float a = (float)lo[n][i] * inv, b = (float)hi[n][i] * inv;
-        if (weight) {
-          a *= weight[wbase + j * 8 + i];
-          b *= weight[wbase + j * 8 + rot_half + i];
-        }
-        const float c = cosrow[j * 8 + i], sn = sinrow[j * 8 + i];
+        const float a = (float)lo[n][i] * inv * wa[i / 4][i % 4], b = (float)hi[n][i] * inv * wb[i / 4][i % 4];
+        const float c = c4[i / 4][i % 4], sn = s4[i / 4][i % 4];
         first[i] = (bf16)(a * c - b * sn);
         second[i] = (bf16)(b * c + a * sn);
       }
@@ -149,13 +155,12 @@ __global__ __launch_bounds__(256) void qkv_norm_prep_vec_kernel(bf16* __restrict
       *(bf16x8*)(dst + j * 8 + rot_half) = second;
     } else {
       const int at = j * 8 + rot_half;
+      floatx4 wa[2];
+#pragma unroll
+      for (int half = 0; half < 2; ++half) wa[half] = weight ? *(const floatx4*)(weight + wbase + at + half * 4) : one4;
       bf16x8 only;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        float a = (float)lo[n][i] * inv;
-        if (weight) a *= weight[wbase + at + i];
-        only[i] = (bf16)a;
-      }
+      for (int i = 0; i < 8; ++i) only[i] = (bf16)((float)lo[n][i] * inv * wa[i / 4][i % 4]);
       *(bf16x8*)(dst + at) = only;
     }
   }
@@ -285,7 +290,8 @@ LRS_API int lrs_qkv_norm_prep(void* qkv, int dtype, int tokens, int row_stride, 
   if (dtype == LRS_F32)
     qkv_norm_prep_kernel<float><<<tokens, 256, 0, s>>>((float*)qkv, row_stride, nq, nkv, d, dv, q_weight, k_weight, eps, cosv, sinv, rot_half,
                                                        (float*)k_pages, (float*)v_pages, slots, page_size);
-  else if (dtype == LRS_BF16 && d % 8 == 0 && rot_half % 8 == 0 && row_stride % 8 == 0 && (uintptr_t)qkv % 16 == 0 &&
+  else if (dtype == LRS_BF16 && d % 8 == 0 && rot_half % 8 == 0 && row_stride % 8 == 0 &&
+           ((uintptr_t)qkv | (uintptr_t)q_weight | (uintptr_t)k_weight | (uintptr_t)cosv | (uintptr_t)sinv) % 16 == 0 &&
            (nq + nkv) * (d - rot_half) / 8 <= 256 * PREP_ITEMS)
     qkv_norm_prep_vec_kernel<<<tokens, 256, 0, s>>>((bf16*)qkv, row_stride, nq, nkv, d, dv, q_weight, k_weight, eps, cosv, sinv, rot_half,
                                                     (bf16*)k_pages, (bf16*)v_pages, slots, page_size);
