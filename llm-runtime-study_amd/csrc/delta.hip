@@ -420,6 +420,34 @@ __global__ __launch_bounds__(256) void ssm_gate_kernel(const float* __restrict__
   const int64_t token = pair / parts;
   const int64_t first = (pair % parts) * part_size, inner = (int64_t)parts * part_size;
   float ss = 0.f;
+  constexpr int HELD = 16;                 // parts of up to 1,024 values stay in registers between the sum and the norm
+  if (part_size <= HELD * WAVE) {
+    float r[HELD], k[HELD], z[HELD];
+#pragma unroll
+    for (int n = 0; n < HELD; ++n) {       // every load is on its way before the first exponential
+      const int i = lane + n * WAVE;
+      if (i < part_size) {
+        r[n] = raw_out[token * inner + first + i];
+        k[n] = skip[token * inner + first + i];
+        z[n] = to_float(proj[token * ld + first + i]);
+      }
+    }
+#pragma unroll
+    for (int n = 0; n < HELD; ++n) {
+      if (lane + n * WAVE < part_size) {
+        r[n] = (r[n] + k[n]) * silu_f(z[n]);
+        ss = fmaf(r[n], r[n], ss);
+      }
+    }
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)part_size + eps);
+#pragma unroll
+    for (int n = 0; n < HELD; ++n) {
+      const int i = lane + n * WAVE;
+      if (i < part_size) out[token * inner + first + i] = from_float<TO>(r[n] * inv * norm_w[first + i]);
+    }
+    return;
+  }
   for (int i = lane; i < part_size; i += WAVE) {
     const float y = (raw_out[token * inner + first + i] + skip[token * inner + first + i]) * silu_f(to_float(proj[token * ld + first + i]));
     ss = fmaf(y, y, ss);

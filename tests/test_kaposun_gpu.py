@@ -89,7 +89,7 @@ def step_through(part, dtype, inputs, width, schedule=SCHEDULE, release_before=(
 # ------------------------------------------------------------------------------------- mechanisms alone
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,groups,state,e,taps,parts", [(4, 2, 24, 40, 3, 2), (2, 2, 64, 64, 4, 1), (3, 1, 128, 16, 2, 3), (1, 1, 10, 7, 1, 1),
-                                                             (6, 3, 48, 32, 4, 6), (2, 1, 256, 8, 5, 4)])
+                                                             (6, 3, 48, 32, 4, 6), (2, 1, 256, 8, 5, 4), (20, 4, 16, 64, 2, 1)])
 def test_state_space_part(dtype, heads, groups, state, e, taps, parts):
     from llm_runtime_study_amd.parts import PartSpec, create
 
