@@ -50,7 +50,7 @@ def napizen_like(shape: dict, layers: int, experts: int = 32, top: int = 8, rank
             "layers": [{"type": "latent_attention", "mixer": mixer, "mlp": routed if index % 2 else dense} for index in range(layers)]}
 
 
-def kaposun_like(shape: dict, layers: int, window: int = 4096, keep_first: int = 4, state: int = 128) -> dict:
+def kaposun_like(shape: dict, layers: int, window: int = 4096, keep_first: int = 8, state: int = 128) -> dict:
     """A Kaposun configuration with the layer sizes of a dense shape above, for measurements beside it: the same width,
     vocabulary, heads and dense feed-forward size (two matrices where the shape has three); in turn a state space layer
     (inner size twice the width in heads of 64 values, `state` numbers a value, 8 groups), an attention layer over the whole
@@ -59,7 +59,7 @@ def kaposun_like(shape: dict, layers: int, window: int = 4096, keep_first: int =
     width, heads, kv_heads, dim = shape["hidden_size"], shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"]
     mlp = {"kind": "dense", "ff": shape["intermediate_size"]}
     sizes = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5}
-    attention = {"type": "attention", "mlp": mlp, "mixer": dict(sizes, rot={"base": 1000000.0, "dims": dim, "scaling": {"factor": 2.0}})}
+    attention = {"type": "attention", "mlp": mlp, "mixer": dict(sizes, rot={"base": 500000.0, "dims": dim, "scaling": {"factor": 4.0}})}
     state_space = {"type": "mamba2", "mlp": mlp, "mixer": {"heads": 2 * width // 64, "groups": 8, "state": state, "vdim": 64, "conv": 4, "norm_groups": 8}}
     pair = {"type": "parallel", "mlp": mlp, "mixer": {"left": dict(sizes, mask={"size": window, "keep_first": keep_first}),
                                                       "right": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "conv": 4},
