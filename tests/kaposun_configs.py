@@ -76,6 +76,14 @@ SELF_LOOP = model(120, 32, 1e-6, 0.5, [
     attention(2, 1, 16, 16, 0.25, rot=(1e4, 16, 8.0), mlp=dense(32)),
     parallel(attention_sizes(4, 4, 8, 12, 0.35, mask=(20, 2)), (2, 2, 16, 16, 3), 0.6, 0.9, mlp=None),
 ], loop=(1, 2, 3))
+# sizes no kernel likes: a width, heads, states and a vocabulary that are multiples of neither 8 nor 16, five taps, 20 query heads
+# on one key group, a rotated part of six dims, more kept positions than the window holds, a loop of one layer run once
+AWKWARD = model(251, 100, 4e-6, 0.45, [
+    mamba(5, 5, 12, 20, 5, 5, mlp=dense(90)),
+    attention(20, 1, 20, 12, 0.22, rot=(3000.0, 6, 1.5), mlp=dense(44)),
+    parallel(attention_sizes(3, 3, 40, 40, 0.16, mask=(6, 11)), (6, 3, 20, 12, 5), 0.9, 1.1, mlp=None),
+    attention(2, 1, 36, 52, 0.17, mlp=dense(60)),
+], loop=(2, 3, 1))
 # wide enough that prompts go through the products for many rows (the vendor library's in bfloat16)
 WIDE = model(1000, 512, 1e-6, 0.25, [
     mamba(8, 2, 64, 64, 4, 2, mlp=dense(512)),

@@ -20,7 +20,7 @@ def test_configuration_reads_back_and_names_its_tensors(tmp_path):
     from llm_runtime_study_amd.models import DecoderModel
     from llm_runtime_study_amd.parts import BothNeeds, PagedKVNeed, StateNeed
 
-    for raw in (configs.ODD, configs.CORES, configs.ONES, configs.SELF_LOOP, configs.WIDE):
+    for raw in (configs.ODD, configs.CORES, configs.ONES, configs.SELF_LOOP, configs.WIDE, configs.AWKWARD):
         config = config_from_dict(raw)
         assert isinstance(config, KaposunConfig) and config.to_json_dict() == raw
         model = DecoderModel(spec_for(config))

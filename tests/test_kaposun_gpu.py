@@ -230,8 +230,9 @@ def test_sum_into_the_stream_leaves_the_next_norm(cols):
 
 
 # ------------------------------------------------------------------------------------- whole models
-MODEL_LENGTHS = {"odd": [1, 5, 23, 64, 97, 130, 33, 16], "cores": [3, 40, 64, 129, 210, 18], "ones": [2, 17, 48, 65, 150, 31, 9], "self_loop": [4, 70, 31, 120, 2]}
-RAW = {"odd": configs.ODD, "cores": configs.CORES, "ones": configs.ONES, "self_loop": configs.SELF_LOOP}
+MODEL_LENGTHS = {"odd": [1, 5, 23, 64, 97, 130, 33, 16], "cores": [3, 40, 64, 129, 210, 18], "ones": [2, 17, 48, 65, 150, 31, 9], "self_loop": [4, 70, 31, 120, 2],
+                 "awkward": [7, 50, 1, 100, 33, 140]}
+RAW = {"odd": configs.ODD, "cores": configs.CORES, "ones": configs.ONES, "self_loop": configs.SELF_LOOP, "awkward": configs.AWKWARD}
 
 
 @pytest.fixture(scope="module")
@@ -311,7 +312,7 @@ def test_whole_then_last_tokens_one_by_one_then_portions(models, name, dtype, tm
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,seed", [("odd", 0), ("odd", 1), ("cores", 2), ("ones", 3), ("self_loop", 4)])
+@pytest.mark.parametrize("name,seed", [("odd", 0), ("odd", 1), ("cores", 2), ("ones", 3), ("self_loop", 4), ("awkward", 6)])
 def test_mixed_steps_with_pages_and_slots_used_again(models, name, seed, dtype, tmp_path):
     folder, raw, requests, want = models[name]
     budget = 2 * max(round64(len(t)) for t in requests.values())
