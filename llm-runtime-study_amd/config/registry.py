@@ -72,9 +72,11 @@ def _load_builtin() -> None:
     _builtin_loaded = True
     from ..models.qwen3 import build_spec
     from ..text.chat import format_qwen3_chat
+    from ..models.felosun import build_spec as build_felosun
     from ..models.kaposun import build_spec as build_kaposun
     from ..models.napizen import build_spec as build_napizen
     from ..models.nobodra import build_spec as build_nobodra
+    from .felosun import FelosunConfig
     from .kaposun import KaposunConfig
     from .napizen import NapizenConfig
     from .nobodra import NobodraConfig
@@ -88,6 +90,8 @@ def _load_builtin() -> None:
         register_architecture(NapizenConfig.ARCHITECTURE, NapizenConfig, build_napizen)      # token ids only as well
     if KaposunConfig.ARCHITECTURE not in _ARCHITECTURES:
         register_architecture(KaposunConfig.ARCHITECTURE, KaposunConfig, build_kaposun)      # token ids only
+    if FelosunConfig.ARCHITECTURE not in _ARCHITECTURES:
+        register_architecture(FelosunConfig.ARCHITECTURE, FelosunConfig, build_felosun)      # token ids only
     import importlib
     import os
 

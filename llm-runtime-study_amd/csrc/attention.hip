@@ -21,6 +21,26 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // before the reference point moves and the accumulators are rescaled.
 constexpr float RESCALE_STEP = 8.0f;
 
+// A cap on the scores: cap * tanh(x / cap), close to x for small |x| and within (-cap, cap) for all.  tanh by one
+// exponential, exact to a few units in the last place of float32 over the whole range.
+__device__ __forceinline__ float capped(float x, float cap) {
+  const float t = x / cap;
+  const float e = __expf(-2.f * fabsf(t));
+  const float r = (1.f - e) / (1.f + e);
+  return cap * (t < 0.f ? -r : r);
+}
+
+// A sink: one more term exp(sink) in a softmax's denominator that has no key and no value.  Given sums that were taken
+// against the reference point `top` (both in powers of two, as every kernel here keeps them), returns the factor for
+// the weighted sums and changes `total` so that factor * sums / total is the softmax with the sink.
+__device__ __forceinline__ float with_sink(float sink2, float top, float& total) {
+  const float m = fmaxf(top, sink2);
+  const float keep = top == -INFINITY ? 0.f : fast_exp2(top - m);
+  total = total * keep + fast_exp2(sink2 - m);
+  return keep;
+}
+constexpr float LOG2E = 1.4426950408889634f;
+
 // ---------------------------------------------------------- generic kernel
 // One workgroup per (query token, query head); any head_dim, values of any size dv up to 4 * threads.  keep_first: with a
 // window, the keys at positions below keep_first stay visible however far back they lie (they keep their positions).
@@ -30,7 +50,7 @@ __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
     const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_request,
     const int* __restrict__ positions, int nq, int nkv, int d, int dv, int page_size, float scale,
-    int window, int keep_first) {
+    int window, int keep_first, const float* __restrict__ sinks, float softcap) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   float* qs = smem;                           // [d]
   float* probs = qs + d + d % 2;              // [THREADS]
@@ -80,6 +100,7 @@ __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
         for (int i = 0; i < d; ++i) dot = fmaf(qs[i], to_float(kr[i]), dot);
       }
       score = dot * scale;
+      if (softcap > 0.f) score = softcap * tanhf(score / softcap);
     }
     const float tile_max = block_max(score, scratch);
     const float new_max = fmaxf(running_max, tile_max);
@@ -120,7 +141,13 @@ __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
     }
     __syncthreads();
   }
-  const float inv = 1.0f / running_sum;
+  float keep = 1.f;
+  if (sinks) {      // one more term in the denominator, with no key and no value
+    const float sink = sinks[head], top = fmaxf(running_max, sink);
+    keep = expf(running_max - top);
+    running_sum = running_sum * keep + expf(sink - top);
+  }
+  const float inv = keep / running_sum;
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
     const int dim = tid + c * THREADS;
@@ -234,7 +261,8 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_bf16_kernel(
     const bf16* __restrict__ q, int q_stride, bf16* __restrict__ k_pages,
     bf16* __restrict__ v_pages, const int* __restrict__ block_table, int table_stride,
     const int* __restrict__ token_request, const int* __restrict__ positions, int nq, int nkv,
-    int page_size, float scale, int window, int splits, int slots, DecodePrep prep) {
+    int page_size, float scale, int window, int splits, int slots, DecodePrep prep, const float* __restrict__ sinks,
+    float softcap) {
   constexpr int DS = D / 32, DB = D / 16, THREADS = WAVES * 64;
   __shared__ float sm_m[WAVES][16], sm_l[WAVES][16];
   __shared__ float sm_o[WAVES][D][16];
@@ -403,7 +431,8 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_bf16_kernel(
       for (int i = 0; i < 4; ++i) {
         const int key = tile * 32 + g * 8 + h * 4 + i;
         const bool valid = key <= pos && key >= lo;
-        s[h][i] = valid ? s[h][i] * scale2 : -INFINITY;
+        const float scaled = softcap > 0.f ? capped(s[h][i] * scale, softcap) * LOG2E : s[h][i] * scale2;
+        s[h][i] = valid ? scaled : -INFINITY;
         tile_max = fmaxf(tile_max, s[h][i]);
       }
     tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
@@ -474,6 +503,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_bf16_kernel(
     }
     const int head = kvh * group + h;
     if (slots <= 1) {
+      if (sinks) acc *= with_sink(sinks[head] * LOG2E, top, total);
       out[(int64_t)token * out_stride + (int64_t)head * D + dim] = (bf16)(acc / total);
     } else {
       const int64_t slot = ((int64_t)token * nq + head) * slots + split;
@@ -491,7 +521,8 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_bf16_kernel(
 // kernel needs a device-wide fence in every workgroup, and on this chip (eight L2s) those fences
 // write back and invalidate whole caches; measured, they cost many times what this kernel does.
 __global__ void attention_merge_kernel(bf16* __restrict__ out, int out_stride, const float* __restrict__ part_o,
-                                       const float* __restrict__ part_ml, int nq, int d, int splits) {
+                                       const float* __restrict__ part_ml, int nq, int d, int splits,
+                                       const float* __restrict__ sinks) {
   const int token = blockIdx.x, head = blockIdx.y;
   const int64_t base = ((int64_t)token * nq + head) * splits;
   // Everything is asked for before anything is used: the partial sums of a split do not wait for its maximum
@@ -523,6 +554,7 @@ __global__ void attention_merge_kernel(bf16* __restrict__ out, int out_stride, c
         acc += o[i] * weight;
       }
     }
+    if (sinks) acc *= with_sink(sinks[head] * LOG2E, top, total);
     out[(int64_t)token * out_stride + (int64_t)head * d + dim] = (bf16)(acc / total);
   }
 }
@@ -533,7 +565,8 @@ __global__ void attention_merge_kernel(bf16* __restrict__ out, int out_stride, c
 // sums are added in split order, as attention_merge_kernel adds them: the same bits.
 template <int SPLITS>
 __global__ __launch_bounds__(256) void attention_merge_wide_kernel(bf16* __restrict__ out, int out_stride, const float* __restrict__ part_o,
-                                                                   const float* __restrict__ part_ml, int64_t quads, int nq, int d) {
+                                                                   const float* __restrict__ part_ml, int64_t quads, int nq, int d,
+                                                                   const float* __restrict__ sinks) {
   const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (e >= quads) return;
   const int per_head = d / 4;
@@ -562,6 +595,11 @@ __global__ __launch_bounds__(256) void attention_merge_wide_kernel(bf16* __restr
     for (int i = 0; i < 4; ++i) acc[i] += o[s][i] * weight;
   }
   const int64_t token = pair / nq, head = pair % nq;
+  if (sinks) {
+    const float keep = with_sink(sinks[head] * LOG2E, top, total);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] *= keep;
+  }
   bf16x4 r;
 #pragma unroll
   for (int i = 0; i < 4; ++i) r[i] = (bf16)(acc[i] / total);
@@ -569,20 +607,20 @@ __global__ __launch_bounds__(256) void attention_merge_wide_kernel(bf16* __restr
 }
 
 static void launch_attention_merge(bf16* out, int out_stride, const float* part_o, const float* part_ml, int tokens, int nq, int d,
-                                   int splits, hipStream_t s) {
+                                   int splits, const float* sinks, hipStream_t s) {
   const bool wide = tokens >= 64 && d % 4 == 0 && out_stride % 4 == 0 && (uintptr_t)out % 8 == 0 && (uintptr_t)part_o % 16 == 0 &&
                     (uintptr_t)part_ml % 8 == 0 && (splits == 2 || splits == 3 || splits == 4 || splits == 5 || splits == 8 || splits == 9);
   if (wide) {
     const int64_t quads = (int64_t)tokens * nq * (d / 4);
     const int blocks = (int)((quads + 255) / 256);
-    if (splits == 2) attention_merge_wide_kernel<2><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d);
-    else if (splits == 3) attention_merge_wide_kernel<3><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d);
-    else if (splits == 4) attention_merge_wide_kernel<4><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d);
-    else if (splits == 5) attention_merge_wide_kernel<5><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d);
-    else if (splits == 9) attention_merge_wide_kernel<9><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d);
-    else attention_merge_wide_kernel<8><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d);
+    if (splits == 2) attention_merge_wide_kernel<2><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d, sinks);
+    else if (splits == 3) attention_merge_wide_kernel<3><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d, sinks);
+    else if (splits == 4) attention_merge_wide_kernel<4><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d, sinks);
+    else if (splits == 5) attention_merge_wide_kernel<5><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d, sinks);
+    else if (splits == 9) attention_merge_wide_kernel<9><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d, sinks);
+    else attention_merge_wide_kernel<8><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d, sinks);
   } else {
-    attention_merge_kernel<<<dim3(tokens, nq), d < 64 ? 64 : d, 0, s>>>(out, out_stride, part_o, part_ml, nq, d, splits);
+    attention_merge_kernel<<<dim3(tokens, nq), d < 64 ? 64 : d, 0, s>>>(out, out_stride, part_o, part_ml, nq, d, splits, sinks);
   }
 }
 
@@ -595,7 +633,7 @@ __global__ __launch_bounds__(WAVE) void attention_kept_bf16_kernel(
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_request,
     const int* __restrict__ positions, int nq, int nkv, int d, int page_size, float scale, int window, int keep_first,
-    int slots, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    int slots, float* __restrict__ part_o, float* __restrict__ part_ml, float softcap) {
   constexpr int PER_LANE = 4;                                     // heads of up to 256 dims
   const int token = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int kvh = head / (nq / nkv);
@@ -627,7 +665,7 @@ __global__ __launch_bounds__(WAVE) void attention_kept_bf16_kernel(
     }
 #pragma unroll
     for (int step = 1; step < WAVE; step *= 2) dot += __shfl_xor(dot, step, WAVE);
-    const float score = dot * scale2;
+    const float score = softcap > 0.f ? capped(dot * scale, softcap) * LOG2E : dot * scale2;
     const float new_top = fmaxf(top, score);
     const float keep = top == -INFINITY ? 0.f : fast_exp2(top - new_top);
     const float weight = fast_exp2(score - new_top);
@@ -650,10 +688,10 @@ __global__ __launch_bounds__(WAVE) void attention_kept_bf16_kernel(
 static void launch_attention_kept(const bf16* q, int q_stride, const bf16* k_pages, const bf16* v_pages, const int* block_table,
                                   int table_stride, const int* token_request, const int* positions, int tokens, int nq, int nkv, int d,
                                   int page_size, float scale, int window, int keep_first, int slots, float* part_o, float* part_ml,
-                                  hipStream_t s) {
+                                  float softcap, hipStream_t s) {
   attention_kept_bf16_kernel<<<dim3(tokens, nq), WAVE, 0, s>>>(q, q_stride, k_pages, v_pages, block_table, table_stride, token_request,
                                                                positions, nq, nkv, d, page_size, scale, window, keep_first, slots, part_o,
-                                                               part_ml);
+                                                               part_ml, softcap);
 }
 
 // Decode step in bf16: one query token per request.  part_o [tokens, nq, splits, d] and part_ml
@@ -669,7 +707,8 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
                                  const int* positions, int tokens, int max_context, int nq, int nkv, int d,
                                  int page_size, float scale, int window, int keep_first, int splits, int form, int prepare,
                                  const void* q_weight, const void* k_weight, int w_dtype, float eps,
-                                 const float* cosv, const float* sinv, int kv_columns, void* stream) {
+                                 const float* cosv, const float* sinv, int kv_columns, const float* sinks, float softcap,
+                                 void* stream) {
   LRS_REQUIRE(tokens > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_decode: bad sizes tokens=%d nq=%d nkv=%d", tokens, nq, nkv);
   LRS_REQUIRE(nq / nkv <= 16, "attention_decode: %d query heads per kv head, at most 16 fit a tile", nq / nkv);
   LRS_REQUIRE(page_size % 16 == 0, "attention_decode: page size %d is not a multiple of 16", page_size);
@@ -678,6 +717,7 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
   const int slots = splits + (keep_first > 0 ? 1 : 0);          // the kept keys' share is one more partial result
   LRS_REQUIRE(splits >= 1 && (slots == 1 || (part_o && part_ml)), "attention_decode: %d partial results need their buffers", slots);
   LRS_REQUIRE(form >= 0 && form <= 2, "attention_decode: form must be 0, 1 or 2, got %d", form);
+  LRS_REQUIRE(softcap >= 0.f, "attention_decode: the cap on the scores must be positive (0 = none), got %g", (double)softcap);
   LRS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0, "attention_decode: q rows must be 16-byte aligned");
   dim3 grid(splits, nkv, tokens);
   hipStream_t s = (hipStream_t)stream;
@@ -701,7 +741,7 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
   // tile on the way while it works (heads of 192 dims have no registers for that and stay with 0)
 #define ARGS                                                                                                 \
   (bf16*)out, out_stride, part_o, part_ml, (const bf16*)q, q_stride, (bf16*)k_pages, (bf16*)v_pages, block_table, \
-      table_stride, token_request, positions, nq, nkv, page_size, scale, window, splits, slots, prep
+      table_stride, token_request, positions, nq, nkv, page_size, scale, window, splits, slots, prep, slots == 1 ? sinks : nullptr, softcap
 #define LAUNCH_PREP(D, PREP)                                                                                 \
   do {                                                                                                       \
     if (form == 2 && D <= 128) attention_decode_bf16_kernel<D, PREP, 8, (D <= 128)><<<grid, 512, table_lds, s>>>(ARGS); \
@@ -727,11 +767,11 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
   if (lrs_check_launch("attention_decode")) return 1;
   if (keep_first > 0) {
     launch_attention_kept((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, token_request,
-                          positions, tokens, nq, nkv, d, page_size, scale, window, keep_first, slots, part_o, part_ml, s);
+                          positions, tokens, nq, nkv, d, page_size, scale, window, keep_first, slots, part_o, part_ml, softcap, s);
     if (lrs_check_launch("attention_kept")) return 1;
   }
   if (slots > 1) {
-    launch_attention_merge((bf16*)out, out_stride, part_o, part_ml, tokens, nq, d, slots, s);
+    launch_attention_merge((bf16*)out, out_stride, part_o, part_ml, tokens, nq, d, slots, sinks, s);
     return lrs_check_launch("attention_merge");
   }
   return 0;
@@ -764,7 +804,8 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_request,
     const int* __restrict__ positions, const int* __restrict__ qblock_token0,
     const int* __restrict__ qblock_count, int n_blocks, int chunk, int nq, int nkv, int page_size, float scale,
-    int window, int splits, int slots, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    int window, int splits, int slots, float* __restrict__ part_o, float* __restrict__ part_ml,
+    const float* __restrict__ sinks, float softcap) {
   constexpr int DS = D / 32, DB = D / 16;
   // Padded LDS rows.  Every fragment is read 16 bytes a lane, 16 rows at a time (the lane's row is col, its
   // piece g), which the LDS serves at its full 256 bytes a cycle when rows lie 32 bytes more than a multiple
@@ -902,6 +943,15 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
 #pragma unroll
           for (int b = 0; b < QB; ++b) sc[b][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kfrag, qf[b][c], sc[b][h], 0, 0, 0);
         }
+      if (softcap > 0.f) {       // the cap, in units of the unscaled scores (the scale enters with the exponent)
+        const float cap = softcap / scale;
+#pragma unroll
+        for (int b = 0; b < QB; ++b)
+#pragma unroll
+          for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sc[b][h][i] = capped(sc[b][h][i], cap);
+      }
     };
     // weights: one step of the running softmax, p = 2^(s * scale2 - reference * scale2) as bfloat16 operands.
     // The reference point of a query's exponentials need not be its maximum: any value that keeps the
@@ -1049,7 +1099,8 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
           part_ml[slot * 2 + 1] = total;
         }
       } else if (live[b]) {
-        const float inv = 1.0f / total;
+        const float keep = sinks ? with_sink(sinks[head] * LOG2E, run_max[b] * scale2, total) : 1.f;
+        const float inv = keep / total;
         bf16* dst = out + (int64_t)(token0 + b * 16 + col) * out_stride + (int64_t)head * D + g * 4;
 #pragma unroll
         for (int e = 0; e < DB; ++e) {
@@ -1090,7 +1141,8 @@ __global__ __launch_bounds__(MANY_WAVES ? 512 : 256, MANY_WAVES ? 1 : 2) void at
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_request,
     const int* __restrict__ positions, const int* __restrict__ qblock_token0,
     const int* __restrict__ qblock_count, int n_blocks, int chunk, int nq, int nkv, int page_size, float scale,
-    int window, int splits, int slots, float* __restrict__ part_o, float* __restrict__ part_ml, int prepare_q, DecodePrep prep) {
+    int window, int splits, int slots, float* __restrict__ part_o, float* __restrict__ part_ml, int prepare_q, DecodePrep prep,
+    const float* __restrict__ sinks) {
   constexpr int D = 128, DS = D / 32, DB = D / 16, STAGES = 3;
   constexpr int KBLOCK = 1024 + 32, KBYTES = 8 * KBLOCK, VHALF = 16 * D * 2 + 16, VBYTES = 2 * VHALF;
   constexpr int VSTAGE = (VBYTES + 63) / 64 * 64;
@@ -1450,7 +1502,8 @@ __global__ __launch_bounds__(MANY_WAVES ? 512 : 256, MANY_WAVES ? 1 : 2) void at
           part_ml[slot * 2 + 1] = total;
         }
       } else if (live[b]) {
-        const float inv = 1.0f / total;
+        const float keep = sinks ? with_sink(sinks[head] * LOG2E, run_max[b] * scale2, total) : 1.f;
+        const float inv = keep / total;
         bf16* dst = out + (int64_t)(token0 + b * 16 + col) * out_stride + (int64_t)head * D + g * 4;
 #pragma unroll
         for (int e = 0; e < DB; ++e) {
@@ -1508,7 +1561,7 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
                                   const int* qblock_count, int n_blocks, int max_count, int max_context, int nq,
                                   int nkv, int d, int page_size, float scale, int window, int keep_first, int tokens, int splits,
                                   float* part_o, float* part_ml, int prepare, const void* q_weight, int w_dtype, float eps,
-                                  const float* cosv, const float* sinv, void* stream) {
+                                  const float* cosv, const float* sinv, const float* sinks, float softcap, void* stream) {
   LRS_REQUIRE(n_blocks > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_prefill: bad sizes blocks=%d nq=%d nkv=%d", n_blocks, nq, nkv);
   if (prepare) {
     LRS_REQUIRE(lrs_attention_prefill_prepares(d), "attention_prefill: only the kernel for heads of 128 prepares the queries itself, got head_dim %d", d);
@@ -1519,10 +1572,13 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
   }
   const DecodePrep prep{q_weight, nullptr, w_dtype == LRS_F32, eps, cosv, sinv, 0};
   LRS_REQUIRE(max_count >= 1 && max_count <= 32, "attention_prefill: query groups hold 1..32 tokens, got %d", max_count);
+  LRS_REQUIRE(softcap >= 0.f, "attention_prefill: the cap on the scores must be positive (0 = none), got %g", (double)softcap);
+  LRS_REQUIRE(!(softcap > 0.f && prepare), "attention_prefill: capped scores come with prepared heads");
   LRS_REQUIRE(page_size % 16 == 0, "attention_prefill: page size %d is not a multiple of 16", page_size);
   LRS_REQUIRE(window >= 0 && keep_first >= 0 && (keep_first == 0 || (window > 0 && !prepare)),
               "attention_prefill: kept first positions (%d) need a window and prepared heads", keep_first);
   const int slots = splits + (keep_first > 0 ? 1 : 0);          // the kept keys' share is one more partial result
+  const float* own_sinks = slots == 1 ? sinks : nullptr;          // with partial results the merge adds the sink
   LRS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && out_stride % 4 == 0 && ((uintptr_t)out % 8) == 0,
               "attention_prefill: q rows must be 16-byte and out rows 8-byte aligned");
   // four waves (with fewer heads in a kv group the spare waves still help to bring tiles in), more only below
@@ -1537,14 +1593,14 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
   const int span = window > 0 && window + 32 + 64 < max_context ? window + 32 + 64 : max_context;
   const size_t table_lds = sizeof(int) * (size_t)(span / page_size + 2);
   // (the kernel for heads of 128 reads the block table with scalar loads and keeps no copy)
-  LRS_REQUIRE(d == 128 || table_lds <= 24 * 1024, "attention_prefill: a context of %d tokens needs more block table entries than fit LDS", max_context);
+  LRS_REQUIRE((d == 128 && softcap == 0.f) || table_lds <= 24 * 1024, "attention_prefill: a context of %d tokens needs more block table entries than fit LDS", max_context);
   hipStream_t s = (hipStream_t)stream;
 #define LAUNCH2(D, QB)                                                                                               \
   attention_prefill_bf16_kernel<D, QB><<<grid, block, table_lds, s>>>((bf16*)out, out_stride, (const bf16*)q, q_stride, \
                                                               (const bf16*)k_pages, (const bf16*)v_pages, block_table, \
                                                               table_stride, token_request, positions, qblock_token0, \
                                                               qblock_count, n_blocks, chunk, nq, nkv, page_size, scale, window, \
-                                                              splits, slots, part_o, part_ml)
+                                                              splits, slots, part_o, part_ml, own_sinks, softcap)
 #define LAUNCH(D)                                \
   if (max_count <= 16) LAUNCH2(D, 1);            \
   else LAUNCH2(D, 2)
@@ -1553,6 +1609,10 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
     case 64: LAUNCH(64); break;
     case 96: LAUNCH(96); break;
     case 128:
+      if (softcap > 0.f) {       // capped scores: the kernel for any head size (the one below weaves the next tile's scores into this tile's weights)
+        LAUNCH(128);
+        break;
+      }
       // head size 128 has a kernel of its own, whose tiles go from memory straight into LDS
       // A kv group of five to eight heads: a wave for every head and one walk over the keys instead of two, while
       // the launch is small (measured, 40 heads on 8: 512 tokens 28.9 -> 19.6 us, 512 tokens after 1,536 88 -> 54 us;
@@ -1564,7 +1624,7 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
         attention_prefill_d128_bf16_kernel<QB, MANY, IDLE><<<grid, block, 0, s>>>(                                                    \
             (bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, \
             token_request, positions, qblock_token0, qblock_count, n_blocks, chunk, nq, nkv, page_size, scale, window, splits, slots, part_o, part_ml, \
-            prepare, prep)
+            prepare, prep, own_sinks)
 #define D128_OF(QB)                                      \
         if (many && idle) D128(QB, true, true);          \
         else if (many) D128(QB, true, false);            \
@@ -1585,11 +1645,11 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
   if (lrs_check_launch("attention_prefill")) return 1;
   if (keep_first > 0) {
     launch_attention_kept((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, token_request,
-                          positions, tokens, nq, nkv, d, page_size, scale, window, keep_first, slots, part_o, part_ml, s);
+                          positions, tokens, nq, nkv, d, page_size, scale, window, keep_first, slots, part_o, part_ml, softcap, s);
     if (lrs_check_launch("attention_kept")) return 1;
   }
   if (slots > 1) {
-    launch_attention_merge((bf16*)out, out_stride, part_o, part_ml, tokens, nq, d, slots, s);
+    launch_attention_merge((bf16*)out, out_stride, part_o, part_ml, tokens, nq, d, slots, sinks, s);
     return lrs_check_launch("attention_merge");
   }
   return 0;
@@ -1603,12 +1663,13 @@ LRS_API int lrs_attention(void* out, int out_stride, const void* q, int q_stride
                           const void* v_pages, const int* block_table, int table_stride,
                           const int* token_request, const int* positions, int dtype, int tokens,
                           int nq, int nkv, int d, int dv, int page_size, float scale, int window, int keep_first,
-                          void* stream) {
+                          const float* sinks, float softcap, void* stream) {
   // value pages [P, nkv, dv, page]; out rows hold nq heads of dv values
   LRS_REQUIRE(tokens > 0 && nq > 0 && nkv > 0 && d > 0 && dv > 0 && page_size > 0, "attention: bad sizes tokens=%d nq=%d nkv=%d d=%d dv=%d page=%d", tokens, nq, nkv, d, dv, page_size);
   LRS_REQUIRE(nq % nkv == 0, "attention: %d query heads do not divide into %d kv heads", nq, nkv);
   LRS_REQUIRE(d <= 512 && dv <= 512, "attention: head sizes %d and %d above the supported 512", d, dv);
   LRS_REQUIRE(window >= 0 && keep_first >= 0, "attention: window and keep_first must be >= 0 (0 = none)");
+  LRS_REQUIRE(softcap >= 0.f, "attention: the cap on the scores must be positive (0 = none), got %g", (double)softcap);
   constexpr int THREADS = 128;
   dim3 grid(tokens, nq);
   const size_t lds = sizeof(float) * (d + d % 2 + THREADS) + (sizeof(int64_t) + sizeof(int)) * THREADS + 16;
@@ -1616,11 +1677,11 @@ LRS_API int lrs_attention(void* out, int out_stride, const void* q, int q_stride
   if (dtype == LRS_F32)
     attention_generic_kernel<float, THREADS><<<grid, THREADS, lds, s>>>(
         (float*)out, out_stride, (const float*)q, q_stride, (const float*)k_pages, (const float*)v_pages,
-        block_table, table_stride, token_request, positions, nq, nkv, d, dv, page_size, scale, window, keep_first);
+        block_table, table_stride, token_request, positions, nq, nkv, d, dv, page_size, scale, window, keep_first, sinks, softcap);
   else if (dtype == LRS_BF16)
     attention_generic_kernel<bf16, THREADS><<<grid, THREADS, lds, s>>>(
         (bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)v_pages,
-        block_table, table_stride, token_request, positions, nq, nkv, d, dv, page_size, scale, window, keep_first);
+        block_table, table_stride, token_request, positions, nq, nkv, d, dv, page_size, scale, window, keep_first, sinks, softcap);
   else
     return lrs_fail("attention: unknown dtype %d", dtype);
   return lrs_check_launch("attention");

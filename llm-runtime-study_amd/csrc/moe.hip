@@ -75,7 +75,8 @@ __device__ __forceinline__ void route_token(const float* __restrict__ logits, in
 //                         choice only; weights: the chosen s divided by their sum (+ 1e-20), times `scale`.  With
 //                         groups > 0 the experts form that many equal groups of neighbours, a group's score is the sum of
 //                         its two largest (s + bias), and only experts of the `keep` best groups can be chosen.
-enum { ROUTE_SOFTMAX_CHOSEN = 0, ROUTE_SIGMOID = 1 };
+//   ROUTE_SIGMOID_SCORES  chosen as under ROUTE_SIGMOID; weights: the chosen s themselves, times `scale` (not divided by their sum)
+enum { ROUTE_SOFTMAX_CHOSEN = 0, ROUTE_SIGMOID = 1, ROUTE_SIGMOID_SCORES = 2 };
 struct RouteRule {
   int kind, groups, keep;
   float scale;
@@ -168,8 +169,12 @@ __device__ __forceinline__ void route_token_sigmoid(const float* __restrict__ lo
     }
   }
   // the same lane wrote them: it reads its own stores
-  if (lane == 0)
+  if (lane == 0 && rule.kind == ROUTE_SIGMOID_SCORES) {
+    if (rule.scale != 1.f)
+      for (int k = 0; k < top; ++k) weights[(int64_t)t * top + k] *= rule.scale;
+  } else if (lane == 0) {
     for (int k = 0; k < top; ++k) weights[(int64_t)t * top + k] = weights[(int64_t)t * top + k] / (total + 1e-20f) * rule.scale;
+  }
 }
 
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ bias,
@@ -177,7 +182,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
                                                         int experts, int top, const RouteRule rule) {
   const int t = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
   if (t >= tokens) return;
-  if (rule.kind == ROUTE_SIGMOID) route_token_sigmoid(logits, ld, bias, ids, weights, t, experts, top, threadIdx.x % WAVE, rule);
+  if (rule.kind != ROUTE_SOFTMAX_CHOSEN) route_token_sigmoid(logits, ld, bias, ids, weights, t, experts, top, threadIdx.x % WAVE, rule);
   else route_token(logits, ld, bias, ids, weights, t, experts, top, threadIdx.x % WAVE);
 }
 
@@ -230,7 +235,7 @@ __global__ __launch_bounds__(1024) void moe_route_align_kernel(const float* __re
                                                                const RouteRule rule) {
   extern __shared__ int shared[];
   for (int t = threadIdx.x / WAVE; t < tokens; t += blockDim.x / WAVE) {
-    if (rule.kind == ROUTE_SIGMOID) route_token_sigmoid(logits, ld, bias, ids, weights, t, experts, top, threadIdx.x % WAVE, rule);
+    if (rule.kind != ROUTE_SOFTMAX_CHOSEN) route_token_sigmoid(logits, ld, bias, ids, weights, t, experts, top, threadIdx.x % WAVE, rule);
     else route_token(logits, ld, bias, ids, weights, t, experts, top, threadIdx.x % WAVE);
   }
   __syncthreads();          // the choices are in memory for every thread of the workgroup
@@ -239,15 +244,33 @@ __global__ __launch_bounds__(1024) void moe_route_align_kernel(const float* __re
 
 // ACT_SILU_PAIRS: the matrix holds, for every feature j, a gate row 2j and an up row 2j + 1; the output has half as many columns,
 // out[:, j] = silu(gate_j) * up_j.  Every kernel below leaves a lane four neighbouring columns, so a lane holds whole pairs.
-enum { ACT_NONE = 0, ACT_RELU_SQUARED = 1, ACT_SILU_PAIRS = 2 };
+// ACT_CLAMPED_PAIRS: the same rows; out[:, j] = g * sigmoid(alpha * g) * (u + 1) with g = min(w * gate_j, limit) and
+// u = clamp(w * up_j, -limit, limit), w the weight of the row's (token, choice) pair where a list of them is given: the
+// expert then runs on w times its input, the products being linear in it.
+enum { ACT_NONE = 0, ACT_RELU_SQUARED = 1, ACT_SILU_PAIRS = 2, ACT_CLAMPED_PAIRS = 3 };
+struct PairAct {
+  const float* pair_weights;   // [pairs], or null for 1
+  float alpha, limit;
+};
 __device__ __forceinline__ float silu_times(float gate, float up) { return gate / (1.0f + expf(-gate)) * up; }
+__device__ __forceinline__ float clamped_times(float gate, float up, float w, const PairAct& pa) {
+  const float g = fminf(w * gate, pa.limit), u = fminf(fmaxf(w * up, -pa.limit), pa.limit);
+  return g / (1.0f + expf(-pa.alpha * g)) * (u + 1.0f);
+}
+__device__ __forceinline__ float pair_times(int act, float gate, float up, float w, const PairAct& pa) {
+  return act == ACT_SILU_PAIRS ? silu_times(gate, up) : clamped_times(gate, up, w, pa);
+}
+__device__ __forceinline__ float weight_of_row(const PairAct& pa, const int* __restrict__ sorted, int row) {
+  return pa.pair_weights ? pa.pair_weights[sorted[row]] : 1.f;
+}
 
 // Any dtype, any shape: a 32 x 64 tile of outputs per workgroup of 256 threads, a thread 2 x 4 of them, each the
 // sum of its products in the order of k.
 template <typename T, typename TO>
 __global__ __launch_bounds__(256) void moe_experts_kernel(TO* __restrict__ out, int ldc, const T* __restrict__ a, int lda,
                                                           const T* __restrict__ w, int n, int k, const int* __restrict__ sorted,
-                                                          const int* __restrict__ tile_expert, int top, int gather, int act, int sub) {
+                                                          const int* __restrict__ tile_expert, int top, int gather, int act, int sub,
+                                                          const PairAct pa) {
   constexpr int TM = 32, TN = 64, TK = 16;
   const int expert = tile_expert[blockIdx.x / sub];       // sub: runs of 32 rows in a tile of the sorted list
   if (expert < 0) return;
@@ -291,13 +314,14 @@ __global__ __launch_bounds__(256) void moe_experts_kernel(TO* __restrict__ out, 
   for (int i = 0; i < 2; ++i) {
     const int m = ty * 2 + i;
     if (row_of[m] < 0) continue;
+    const float pw = act == ACT_CLAMPED_PAIRS ? weight_of_row(pa, sorted, row0 + m) : 1.f;
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
       const int c = col0 + tx * 4 + jj;
       if (c >= n) continue;
       float v = acc[i][jj];
-      if (act == ACT_SILU_PAIRS) {
-        if (jj % 2 == 0) out[(int64_t)(row0 + m) * ldc + c / 2] = from_float<TO>(silu_times(v, acc[i][jj + 1]));
+      if (act >= ACT_SILU_PAIRS) {
+        if (jj % 2 == 0) out[(int64_t)(row0 + m) * ldc + c / 2] = from_float<TO>(pair_times(act, v, acc[i][jj + 1], pw, pa));
         continue;
       }
       if (act == ACT_RELU_SQUARED) v = v > 0.f ? v * v : 0.f;
@@ -317,7 +341,7 @@ constexpr int GM = 32, GN = 128, GK = 64, GPAD = 8;
 template <typename TO, int NT>
 __global__ __launch_bounds__(256) void moe_experts_bf16_kernel(TO* __restrict__ out, int ldc, const bf16* __restrict__ a, int lda,
                                                                const bf16* __restrict__ w, int n, int k, const int* __restrict__ sorted,
-                                                               const int* __restrict__ tile_expert, int top, int gather, int act) {
+                                                               const int* __restrict__ tile_expert, int top, int gather, int act, const PairAct pa) {
   const int expert = tile_expert[blockIdx.x];
   if (expert < 0) return;
   __shared__ __attribute__((aligned(16))) bf16 a_s[GM][GK + GPAD];
@@ -377,6 +401,7 @@ __global__ __launch_bounds__(256) void moe_experts_bf16_kernel(TO* __restrict__ 
   for (int i = 0; i < 2; ++i) {
     const int m = i * 16 + lane % 16;
     if (row_of[m] < 0) continue;
+    const float pw = act == ACT_CLAMPED_PAIRS ? weight_of_row(pa, sorted, row0 + m) : 1.f;
 #pragma unroll
     for (int jj = 0; jj < WN; ++jj) {
       const int c = col0 + wave * 16 * WN + jj * 16 + (lane / 16) * 4;
@@ -384,8 +409,8 @@ __global__ __launch_bounds__(256) void moe_experts_bf16_kernel(TO* __restrict__ 
       for (int x = 0; x < 4; ++x) {
         if (c + x >= n) continue;
         float v = acc[i][jj][x];
-        if (act == ACT_SILU_PAIRS) {
-          if (x % 2 == 0) out[(int64_t)(row0 + m) * ldc + (c + x) / 2] = from_float<TO>(silu_times(v, acc[i][jj][x + 1]));
+        if (act >= ACT_SILU_PAIRS) {
+          if (x % 2 == 0) out[(int64_t)(row0 + m) * ldc + (c + x) / 2] = from_float<TO>(pair_times(act, v, acc[i][jj][x + 1], pw, pa));
           continue;
         }
         if (act == ACT_RELU_SQUARED) v = v > 0.f ? v * v : 0.f;
@@ -402,7 +427,7 @@ constexpr int WM = 128;
 template <typename TO>
 __global__ __launch_bounds__(256) void moe_experts_bf16_wide_kernel(TO* __restrict__ out, int ldc, const bf16* __restrict__ a, int lda,
                                                                     const bf16* __restrict__ w, int n, int k, const int* __restrict__ sorted,
-                                                                    const int* __restrict__ tile_expert, int top, int gather, int act) {
+                                                                    const int* __restrict__ tile_expert, int top, int gather, int act, const PairAct pa) {
   // Workgroups are dealt to the chip's eight dies in turn, each with an L2 of its own: number the tiles so that a die
   // gets neighbours (row tiles of one expert under one column tile, which share the weights).
   const int total = gridDim.x * gridDim.y, flat = blockIdx.y * gridDim.x + blockIdx.x;
@@ -468,6 +493,7 @@ __global__ __launch_bounds__(256) void moe_experts_bf16_wide_kernel(TO* __restri
   for (int i = 0; i < 4; ++i) {
     const int m = wm * 64 + i * 16 + lane % 16;
     if (row_of[m] < 0) continue;
+    const float pw = act == ACT_CLAMPED_PAIRS ? weight_of_row(pa, sorted, row0 + m) : 1.f;
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
       const int c = col0 + wn * 64 + jj * 16 + (lane / 16) * 4;
@@ -475,8 +501,8 @@ __global__ __launch_bounds__(256) void moe_experts_bf16_wide_kernel(TO* __restri
       for (int x = 0; x < 4; ++x) {
         if (c + x >= n) continue;
         float v = acc[i][jj][x];
-        if (act == ACT_SILU_PAIRS) {
-          if (x % 2 == 0) out[(int64_t)(row0 + m) * ldc + (c + x) / 2] = from_float<TO>(silu_times(v, acc[i][jj][x + 1]));
+        if (act >= ACT_SILU_PAIRS) {
+          if (x % 2 == 0) out[(int64_t)(row0 + m) * ldc + (c + x) / 2] = from_float<TO>(pair_times(act, v, acc[i][jj][x + 1], pw, pa));
           continue;
         }
         if (act == ACT_RELU_SQUARED) v = v > 0.f ? v * v : 0.f;
@@ -497,7 +523,7 @@ template <typename TO>
 __global__ __launch_bounds__(256, 2) void moe_experts_bf16_fetch_kernel(TO* __restrict__ out, int ldc, const bf16* __restrict__ x, int lda,
                                                                         const bf16* __restrict__ w, int n, int k, const int* __restrict__ sorted,
                                                                         const int* __restrict__ tile_expert, int tiles_m, int tiles_n, int top,
-                                                                        int gather, int act) {
+                                                                        int gather, int act, const PairAct pa) {
   constexpr int BM = 128, BN = 256, BK = 32, STAGES = 3;
   constexpr int XL = BM / 16 / 4, WL = BN / 16 / 4;
   constexpr int STAGE_ELEMENTS = (BM + BN) * BK;
@@ -577,6 +603,7 @@ __global__ __launch_bounds__(256, 2) void moe_experts_bf16_fetch_kernel(TO* __re
   for (int jt = 0; jt < 4; ++jt) {
     const int at = m0_opaque + wm + jt * 16 + r;
     const bool in_use = sorted[at] >= 0;
+    const float pw = in_use && act == ACT_CLAMPED_PAIRS ? weight_of_row(pa, sorted, at) : 1.f;
     const int64_t row_at = (int64_t)at * ldc;
 #pragma unroll
     for (int it = 0; it < 8; ++it) {
@@ -589,8 +616,8 @@ __global__ __launch_bounds__(256, 2) void moe_experts_bf16_fetch_kernel(TO* __re
 #pragma unroll
           for (int i = 0; i < 4; ++i) v[i] = v[i] > 0.f ? v[i] * v[i] : 0.f;
         }
-        if (act == ACT_SILU_PAIRS) {
-          const float first = silu_times(v[0], v[1]), second = silu_times(v[2], v[3]);
+        if (act >= ACT_SILU_PAIRS) {
+          const float first = pair_times(act, v[0], v[1], pw, pa), second = pair_times(act, v[2], v[3], pw, pa);
           if constexpr (sizeof(TO) == 2) *(bf16x2*)((bf16*)out + row_at + row0 / 2) = bf16x2{(bf16)first, (bf16)second};
           else ((float*)out)[row_at + row0 / 2] = first, ((float*)out)[row_at + row0 / 2 + 1] = second;
         } else if constexpr (sizeof(TO) == 2) *(bf16x4*)((bf16*)out + row_at + row0) = bf16x4{(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
@@ -611,13 +638,13 @@ template <typename TW>
 __global__ __launch_bounds__(1024) void moe_combine_kernel(float* __restrict__ residual, const float* __restrict__ rows, int hidden,
                                                            const int* __restrict__ place, const float* __restrict__ weights, int top,
                                                            const TW* __restrict__ norm_w, float eps, bf16* __restrict__ rounded, int kind,
-                                                           float alpha) {
+                                                           float alpha, const float* __restrict__ extra) {
   extern __shared__ float sum[];        // [hidden], 16 floats for the reduction, then the token's rows and weights [top] each
   float* share = sum + hidden + 16;
   int* where = (int*)(share + top);
   const int t = blockIdx.x;
   for (int c = threadIdx.x; c < top; c += blockDim.x) {
-    share[c] = weights[(int64_t)t * top + c];
+    share[c] = weights ? weights[(int64_t)t * top + c] : 1.f;
     where[c] = place[(int64_t)t * top + c];
   }
   __syncthreads();
@@ -626,6 +653,7 @@ __global__ __launch_bounds__(1024) void moe_combine_kernel(float* __restrict__ r
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float acc = 0.f;
     for (int c = 0; c < top; ++c) acc = fmaf(share[c], rows[(int64_t)where[c] * hidden + i], acc);
+    if (extra) acc += extra[(int64_t)t * hidden + i];          // what a part that runs for every token gave out
     if (kind == COMBINE_LAYERNORM) {
       acc = fmaf(alpha, out[i], acc);
       ss += acc;                        // the sum of the row, for its mean
@@ -678,7 +706,7 @@ LRS_API int lrs_moe_max_tiles(int pairs, int experts) {
 }
 
 static int check_rule(const char* who, int kind, int groups, int keep, float scale, int experts, int top) {
-  LRS_REQUIRE(kind == ROUTE_SOFTMAX_CHOSEN || kind == ROUTE_SIGMOID, "%s: unknown routing rule %d", who, kind);
+  LRS_REQUIRE(kind >= ROUTE_SOFTMAX_CHOSEN && kind <= ROUTE_SIGMOID_SCORES, "%s: unknown routing rule %d", who, kind);
   if (kind == ROUTE_SOFTMAX_CHOSEN) {
     LRS_REQUIRE(groups == 0, "%s: groups of experts come with the sigmoid rule only", who);
     return 0;
@@ -732,12 +760,16 @@ LRS_API int lrs_moe_route_align(const float* logits, int ld, const float* bias, 
 // out [max_tiles * tile, n] = rows of `a` (row pair / top of the sorted list if `gather`, else the sorted row
 // itself) times the tile's expert matrix w[expert] [n, k], transposed; act 1: the square of relu; act 2: see ACT_SILU_PAIRS (out has n / 2 columns).
 LRS_API int lrs_moe_experts(void* out, int out_dtype, int ldc, const void* a, const void* w, int dtype, int lda, int n, int k,
-                            const int* sorted, const int* tile_expert, int max_tiles, int tile, int top, int gather, int act, void* stream) {
+                            const int* sorted, const int* tile_expert, int max_tiles, int tile, int top, int gather, int act,
+                            const float* pair_weights, float act_alpha, float act_limit, void* stream) {
+  const PairAct pa{pair_weights, act_alpha, act_limit};
   LRS_REQUIRE(tile == GM || tile == WM, "moe_experts: tiles have %d or %d rows, got %d", GM, WM, tile);
   LRS_REQUIRE(max_tiles > 0 && n > 0 && k > 0 && top > 0, "moe_experts: bad sizes tiles=%d n=%d k=%d top=%d", max_tiles, n, k, top);
-  LRS_REQUIRE(act == ACT_NONE || act == ACT_RELU_SQUARED || act == ACT_SILU_PAIRS, "moe_experts: unknown activation %d", act);
-  LRS_REQUIRE(lda >= k && ldc >= (act == ACT_SILU_PAIRS ? n / 2 : n), "moe_experts: strides lda=%d ldc=%d too small for k=%d n=%d", lda, ldc, k, n);
-  LRS_REQUIRE(act != ACT_SILU_PAIRS || n % 4 == 0, "moe_experts: pairs of gate and up rows come four rows at a time, got %d rows", n);
+  LRS_REQUIRE(act >= ACT_NONE && act <= ACT_CLAMPED_PAIRS, "moe_experts: unknown activation %d", act);
+  LRS_REQUIRE(act != ACT_CLAMPED_PAIRS || act_limit > 0.f, "moe_experts: the clamp's limit must be positive, got %g", (double)act_limit);
+  LRS_REQUIRE(act == ACT_CLAMPED_PAIRS || pair_weights == nullptr, "moe_experts: weights on the inputs come with the clamped activation");
+  LRS_REQUIRE(lda >= k && ldc >= (act >= ACT_SILU_PAIRS ? n / 2 : n), "moe_experts: strides lda=%d ldc=%d too small for k=%d n=%d", lda, ldc, k, n);
+  LRS_REQUIRE(act < ACT_SILU_PAIRS || n % 4 == 0, "moe_experts: pairs of gate and up rows come four rows at a time, got %d rows", n);
   hipStream_t s = (hipStream_t)stream;
   const bool cores = dtype == LRS_BF16 && k % GK == 0 && lda % 8 == 0 && ((uintptr_t)a % 16) == 0 && ((uintptr_t)w % 16) == 0;
   // large steps of shapes the fetching kernel takes: whole slices of 32 of K, rows of the output 16 bytes aligned, offsets
@@ -747,9 +779,9 @@ LRS_API int lrs_moe_experts(void* out, int out_dtype, int ldc, const void* a, co
   if (fetching) {
     const int tiles_n = (n + 255) / 256;
     if (out_dtype == LRS_BF16)
-      moe_experts_bf16_fetch_kernel<bf16><<<max_tiles * tiles_n, 256, 0, s>>>((bf16*)out, ldc, (const bf16*)a, lda, (const bf16*)w, n, k, sorted, tile_expert, max_tiles, tiles_n, top, gather, act);
+      moe_experts_bf16_fetch_kernel<bf16><<<max_tiles * tiles_n, 256, 0, s>>>((bf16*)out, ldc, (const bf16*)a, lda, (const bf16*)w, n, k, sorted, tile_expert, max_tiles, tiles_n, top, gather, act, pa);
     else if (out_dtype == LRS_F32)
-      moe_experts_bf16_fetch_kernel<float><<<max_tiles * tiles_n, 256, 0, s>>>((float*)out, ldc, (const bf16*)a, lda, (const bf16*)w, n, k, sorted, tile_expert, max_tiles, tiles_n, top, gather, act);
+      moe_experts_bf16_fetch_kernel<float><<<max_tiles * tiles_n, 256, 0, s>>>((float*)out, ldc, (const bf16*)a, lda, (const bf16*)w, n, k, sorted, tile_expert, max_tiles, tiles_n, top, gather, act, pa);
     else
       return lrs_fail("moe_experts: unknown output dtype %d", out_dtype);
     return lrs_check_launch("moe_experts");
@@ -757,9 +789,9 @@ LRS_API int lrs_moe_experts(void* out, int out_dtype, int ldc, const void* a, co
   if (cores && tile == WM) {
     dim3 grid(max_tiles, (n + GN - 1) / GN);
     if (out_dtype == LRS_BF16)
-      moe_experts_bf16_wide_kernel<bf16><<<grid, 256, 0, s>>>((bf16*)out, ldc, (const bf16*)a, lda, (const bf16*)w, n, k, sorted, tile_expert, top, gather, act);
+      moe_experts_bf16_wide_kernel<bf16><<<grid, 256, 0, s>>>((bf16*)out, ldc, (const bf16*)a, lda, (const bf16*)w, n, k, sorted, tile_expert, top, gather, act, pa);
     else if (out_dtype == LRS_F32)
-      moe_experts_bf16_wide_kernel<float><<<grid, 256, 0, s>>>((float*)out, ldc, (const bf16*)a, lda, (const bf16*)w, n, k, sorted, tile_expert, top, gather, act);
+      moe_experts_bf16_wide_kernel<float><<<grid, 256, 0, s>>>((float*)out, ldc, (const bf16*)a, lda, (const bf16*)w, n, k, sorted, tile_expert, top, gather, act, pa);
     else
       return lrs_fail("moe_experts: unknown output dtype %d", out_dtype);
     return lrs_check_launch("moe_experts");
@@ -768,7 +800,7 @@ LRS_API int lrs_moe_experts(void* out, int out_dtype, int ldc, const void* a, co
     // few tiles (single tokens, short portions): 64 columns a workgroup, so that twice as many stream the weights
     const bool narrow = (int64_t)max_tiles * ((n + GN - 1) / GN) < 4 * lrs_compute_units();
     dim3 grid(max_tiles, narrow ? (n + 63) / 64 : (n + GN - 1) / GN);
-#define CORES(TO, NT) moe_experts_bf16_kernel<TO, NT><<<grid, 256, 0, s>>>((TO*)out, ldc, (const bf16*)a, lda, (const bf16*)w, n, k, sorted, tile_expert, top, gather, act)
+#define CORES(TO, NT) moe_experts_bf16_kernel<TO, NT><<<grid, 256, 0, s>>>((TO*)out, ldc, (const bf16*)a, lda, (const bf16*)w, n, k, sorted, tile_expert, top, gather, act, pa)
     if (out_dtype == LRS_BF16) { if (narrow) CORES(bf16, 64); else CORES(bf16, 128); }
     else if (out_dtype == LRS_F32) { if (narrow) CORES(float, 64); else CORES(float, 128); }
     else return lrs_fail("moe_experts: unknown output dtype %d", out_dtype);
@@ -776,7 +808,7 @@ LRS_API int lrs_moe_experts(void* out, int out_dtype, int ldc, const void* a, co
     return lrs_check_launch("moe_experts");
   }
   dim3 grid(max_tiles * (tile / GM), (n + 63) / 64);       // the any-shape form walks a tile of 128 rows as four of 32
-#define RUN(T, TO) moe_experts_kernel<T, TO><<<grid, 256, 0, s>>>((TO*)out, ldc, (const T*)a, lda, (const T*)w, n, k, sorted, tile_expert, top, gather, act, tile / GM)
+#define RUN(T, TO) moe_experts_kernel<T, TO><<<grid, 256, 0, s>>>((TO*)out, ldc, (const T*)a, lda, (const T*)w, n, k, sorted, tile_expert, top, gather, act, tile / GM, pa)
   if (dtype == LRS_F32 && out_dtype == LRS_F32) RUN(float, float);
   else if (dtype == LRS_BF16 && out_dtype == LRS_BF16) RUN(bf16, bf16);
   else if (dtype == LRS_BF16 && out_dtype == LRS_F32) RUN(bf16, float);
@@ -786,9 +818,11 @@ LRS_API int lrs_moe_experts(void* out, int out_dtype, int ldc, const void* a, co
 }
 
 // residual [tokens, hidden] += (norm of) sum_c weights[t, c] * rows[place[t, c]]; norm_w null: the plain sum; rounded:
-// where the updated rows are left in bfloat16 as well, or null.
+// where the updated rows are left in bfloat16 as well, or null.  weights null: every choice counts once.  extra [tokens, hidden]
+// (or null): rows added to the sum before the norm.
 LRS_API int lrs_moe_combine(float* residual, const float* rows, int tokens, int hidden, const int* place, const float* weights,
-                            int top, const void* norm_w, int norm_dtype, float eps, void* rounded, int layer_norm, float alpha, void* stream) {
+                            int top, const void* norm_w, int norm_dtype, float eps, void* rounded, int layer_norm, float alpha,
+                            const float* extra, void* stream) {
   // layer_norm (with a norm weight): the stream becomes the layer norm of alpha * stream + sum, instead of taking the sum's RMS norm on top
   LRS_REQUIRE(tokens > 0 && hidden > 0 && top > 0, "moe_combine: bad sizes tokens=%d hidden=%d top=%d", tokens, hidden, top);
   LRS_REQUIRE(!norm_w || eps > 0.f, "moe_combine: eps must be positive");
@@ -799,8 +833,8 @@ LRS_API int lrs_moe_combine(float* residual, const float* rows, int tokens, int 
   hipStream_t s = (hipStream_t)stream;
   const int threads = hidden >= 2048 ? 1024 : 256;
   if (norm_w && norm_dtype == LRS_BF16)
-    moe_combine_kernel<bf16><<<tokens, threads, lds, s>>>(residual, rows, hidden, place, weights, top, (const bf16*)norm_w, eps, (bf16*)rounded, kind, alpha);
+    moe_combine_kernel<bf16><<<tokens, threads, lds, s>>>(residual, rows, hidden, place, weights, top, (const bf16*)norm_w, eps, (bf16*)rounded, kind, alpha, extra);
   else
-    moe_combine_kernel<float><<<tokens, threads, lds, s>>>(residual, rows, hidden, place, weights, top, (const float*)norm_w, eps, (bf16*)rounded, kind, alpha);
+    moe_combine_kernel<float><<<tokens, threads, lds, s>>>(residual, rows, hidden, place, weights, top, (const float*)norm_w, eps, (bf16*)rounded, kind, alpha, extra);
   return lrs_check_launch("moe_combine");
 }

@@ -5,7 +5,7 @@
 //                   whole q part and of the whole k part (one sum of squares each, a weight per column), the half-split
 //                   rotation of the first 2*rot_half dims of every q and k head, q written back in place, k into the
 //                   key pages [page, kv_head, slot, d], v into the value pages [page, kv_head, dv, slot];
-//   sigmoid_gate    out[t, c] *= sigmoid(gate[t, c]): the output gate of the heads;
+//   sigmoid_gate    out[t, c] *= sigmoid(gate[t, c / group]): the output gate of the heads, a value a column or one a head;
 //   axpby           out = alpha * a + beta * b over float32 rows: sums of sublayer outputs and the scaled residual add,
 //                   optionally followed by the RMS norm of the new rows (the next layer's input) in the same pass;
 //   activation      out = act(x) elementwise: exact (erf) gelu, tanh gelu, silu, relu.
@@ -173,11 +173,12 @@ __global__ __launch_bounds__(256) void qkv_norm_prep_vec_kernel(bf16* __restrict
 }
 
 template <typename T>
-__global__ void sigmoid_gate_kernel(T* __restrict__ out, int out_stride, const T* __restrict__ gate, int gate_stride, int rows, int cols) {
+__global__ void sigmoid_gate_kernel(T* __restrict__ out, int out_stride, const T* __restrict__ gate, int gate_stride, int rows, int cols,
+                                    int group) {
   const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (e >= (int64_t)rows * cols) return;
   const int64_t r = e / cols, c = e % cols;
-  const float g = to_float(gate[r * gate_stride + c]);
+  const float g = to_float(gate[r * gate_stride + c / group]);     // one gate value for every `group` neighbouring columns
   T* o = out + r * out_stride + c;
   *o = from_float<T>(to_float(*o) / (1.f + expf(-g)));
 }
@@ -302,13 +303,14 @@ LRS_API int lrs_qkv_norm_prep(void* qkv, int dtype, int tokens, int row_stride, 
   return lrs_check_launch("qkv_norm_prep");
 }
 
-LRS_API int lrs_sigmoid_gate(void* out, int out_stride, const void* gate, int gate_stride, int dtype, int rows, int cols, void* stream) {
-  LRS_REQUIRE(rows > 0 && cols > 0 && out_stride >= cols && gate_stride >= cols, "sigmoid_gate: bad sizes rows=%d cols=%d", rows, cols);
+LRS_API int lrs_sigmoid_gate(void* out, int out_stride, const void* gate, int gate_stride, int dtype, int rows, int cols, int group, void* stream) {
+  LRS_REQUIRE(rows > 0 && cols > 0 && group > 0 && cols % group == 0 && out_stride >= cols && gate_stride >= cols / group,
+              "sigmoid_gate: bad sizes rows=%d cols=%d group=%d", rows, cols, group);
   const int64_t count = (int64_t)rows * cols;
   const unsigned blocks = (unsigned)((count + 255) / 256);
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == LRS_F32) sigmoid_gate_kernel<float><<<blocks, 256, 0, s>>>((float*)out, out_stride, (const float*)gate, gate_stride, rows, cols);
-  else if (dtype == LRS_BF16) sigmoid_gate_kernel<bf16><<<blocks, 256, 0, s>>>((bf16*)out, out_stride, (const bf16*)gate, gate_stride, rows, cols);
+  if (dtype == LRS_F32) sigmoid_gate_kernel<float><<<blocks, 256, 0, s>>>((float*)out, out_stride, (const float*)gate, gate_stride, rows, cols, group);
+  else if (dtype == LRS_BF16) sigmoid_gate_kernel<bf16><<<blocks, 256, 0, s>>>((bf16*)out, out_stride, (const bf16*)gate, gate_stride, rows, cols, group);
   else return lrs_fail("sigmoid_gate: unknown dtype %d", dtype);
   return lrs_check_launch("sigmoid_gate");
 }

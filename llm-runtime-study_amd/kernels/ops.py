@@ -124,10 +124,15 @@ _SIGNATURES = {
                                             c_void_p, c_int64, c_void_p]),
     "lrs_norm_begin_parts": (c_int, [c_int]),
     "lrs_attention": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
-                              c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p]),
+                              c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_float, c_void_p]),
     "lrs_qkv_norm_prep": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
                                   c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
-    "lrs_sigmoid_gate": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    "lrs_sigmoid_gate": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "lrs_rotate_unit_prep": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p, c_int, c_int,
+                                     c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    "lrs_gated_clamped": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_void_p]),
+    "lrs_add_gathered": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p]),
+    "lrs_scale_values": (c_int, [c_void_p, c_int64, c_float, c_void_p]),
     "lrs_axpby": (c_int, [c_void_p, c_void_p, c_float, c_void_p, c_float, c_int, c_int, c_void_p, c_float, c_void_p, c_int, c_void_p]),
     "lrs_activation": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int, c_void_p]),
     "lrs_delta_rule_channels": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
@@ -138,10 +143,10 @@ _SIGNATURES = {
                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "lrs_attention_decode": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                      c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int,
-                                     c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_void_p]),
+                                     c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_void_p, c_float, c_void_p]),
     "lrs_attention_prefill": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                                       c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
-                                      c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p]),
+                                      c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_float, c_void_p]),
     "lrs_attention_prefill_prepares": (c_int, [c_int]),
     "lrs_compute_units": (c_int, []),
     "lrs_gemm_lines_width": (c_int, [c_int, c_int, c_int]),
@@ -167,7 +172,7 @@ _SIGNATURES = {
                                     c_int, c_int, c_int, c_float, c_void_p]),
     "lrs_moe_align": (c_int, [c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_moe_experts": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
-                                c_int, c_int, c_void_p]),
+                                c_int, c_int, c_void_p, c_float, c_float, c_void_p]),
     "lrs_layernorm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_void_p]),
     "lrs_scale_add_layernorm": (c_int, [c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_int, c_float, c_void_p, c_void_p]),
     "lrs_soft_cap": (c_int, [c_void_p, c_int64, c_float, c_void_p]),
@@ -180,7 +185,7 @@ _SIGNATURES = {
     "lrs_head_gemm": (c_int, [c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "lrs_latent_attention": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                      c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
-    "lrs_moe_combine": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_int, c_float, c_void_p]),
+    "lrs_moe_combine": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_int, c_float, c_void_p, c_void_p]),
 }
 
 
@@ -216,11 +221,11 @@ def library():
 #
 # PLAN_OPS fixes the number of each entry point inside a plan; csrc/plan_dispatch.inc, made from this list
 # and _SIGNATURES by kernels/plan_codegen.py, is the other side (a test keeps the two in step).
-PLAN_OPS = ("lrs_activation", "lrs_add_into", "lrs_add_rmsnorm", "lrs_advance_decode", "lrs_advance_slots", "lrs_attention", "lrs_attention_decode",
+PLAN_OPS = ("lrs_activation", "lrs_add_gathered", "lrs_add_into", "lrs_add_rmsnorm", "lrs_advance_decode", "lrs_advance_slots", "lrs_attention", "lrs_attention_decode",
             "lrs_attention_prefill", "lrs_axpby", "lrs_choose_tokens", "lrs_choose_tokens_split", "lrs_copy_to_pinned", "lrs_delta_rule", "lrs_delta_rule_channels", "lrs_embed", "lrs_fill_i32",
-            "lrs_filter_logits", "lrs_gather_rows", "lrs_gemm", "lrs_gemm_lines_add_rmsnorm", "lrs_gemm_mid_add_norm_begin", "lrs_gemm_mid_qk_prep", "lrs_gemm_mid_scaled",
+            "lrs_filter_logits", "lrs_gated_clamped", "lrs_gather_rows", "lrs_gemm", "lrs_gemm_lines_add_rmsnorm", "lrs_gemm_mid_add_norm_begin", "lrs_gemm_mid_qk_prep", "lrs_gemm_mid_scaled",
             "lrs_gemm_norm_chain", "lrs_head_gemm", "lrs_latent_attention", "lrs_latent_attention_groups", "lrs_latent_prep", "lrs_layernorm", "lrs_library_gemm", "lrs_moe_align", "lrs_moe_combine", "lrs_moe_experts", "lrs_moe_route", "lrs_moe_route_align", "lrs_norm_add",
-            "lrs_qk_prep", "lrs_qkv_norm_prep", "lrs_rmsnorm", "lrs_rope_table", "lrs_round_rows", "lrs_scale_add_layernorm", "lrs_scale_rows", "lrs_sigmoid_gate", "lrs_silu_mul", "lrs_soft_cap", "lrs_ssm")
+            "lrs_qk_prep", "lrs_qkv_norm_prep", "lrs_rmsnorm", "lrs_rope_table", "lrs_rotate_unit_prep", "lrs_round_rows", "lrs_scale_add_layernorm", "lrs_scale_rows", "lrs_scale_values", "lrs_sigmoid_gate", "lrs_silu_mul", "lrs_soft_cap", "lrs_ssm")
 _PLAN_INDEX = {name: index for index, name in enumerate(PLAN_OPS)}
 
 
@@ -960,10 +965,20 @@ def scale_rows(out: torch.Tensor, x: torch.Tensor, sumsq: torch.Tensor, eps: flo
 
 
 # -------------------------------------------------------------- attention
+def _sinks(sinks: torch.Tensor | None, nq: int, who: str):
+    if sinks is None:
+        return None
+    _need(sinks.dtype == torch.float32 and sinks.numel() == nq and sinks.is_contiguous(), f"{who}: sinks must be float32 [{nq}]")
+    return _dev(sinks, "sinks")
+
+
 def attention(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
-              token_request: torch.Tensor, positions: torch.Tensor, nq: int, scale: float, window: int = 0, keep_first: int = 0) -> None:
+              token_request: torch.Tensor, positions: torch.Tensor, nq: int, scale: float, window: int = 0, keep_first: int = 0,
+              sinks: torch.Tensor | None = None, softcap: float = 0.0) -> None:
     """out [T, nq*dv]; q [T, >= nq*d] (leading nq*d columns of each row); key pages [P, nkv, page, d],
-    value pages [P, nkv, dv, page].  window: a token at p sees keys above p - window; keep_first: and those below keep_first."""
+    value pages [P, nkv, dv, page].  window: a token at p sees keys above p - window; keep_first: and those below keep_first.
+    sinks (float32 [nq]): the softmax's denominator of head h has one more term exp(sinks[h]), without key or value.
+    softcap > 0: the scaled scores pass softcap * tanh(score / softcap) before the softmax."""
     tokens = out.shape[0]
     _need(k_pages.dim() == 4 and v_pages.dim() == 4 and k_pages.is_contiguous() and v_pages.is_contiguous(), "attention: pages must be contiguous")
     _, nkv, page_size, d = k_pages.shape
@@ -977,7 +992,7 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages
     _launch("lrs_attention", 
         _dev(out, "out"), _rows(out, "out"), _dev(q, "q"), _rows(q, "q"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"),
         _dev(block_table, "block_table"), block_table.stride(0), _dev(token_request, "token_request"), _dev(positions, "positions"),
-        dtype_code(q.dtype), tokens, nq, nkv, d, dv, page_size, scale, window, keep_first, _stream())
+        dtype_code(q.dtype), tokens, nq, nkv, d, dv, page_size, scale, window, keep_first, _sinks(sinks, nq, "attention"), float(softcap), _stream())
 
 
 def qkv_norm_prep(qkv: torch.Tensor, nq: int, nkv: int, d: int, dv: int, q_weight, k_weight, eps: float, cos, sin,
@@ -1008,10 +1023,60 @@ def qkv_norm_prep(qkv: torch.Tensor, nq: int, nkv: int, d: int, dv: int, q_weigh
 
 
 def sigmoid_gate(out: torch.Tensor, gate: torch.Tensor) -> None:
-    """out *= sigmoid(gate), both [T, C] with rows that may be strided (a gate that lies in a wider projection row)."""
-    _need(out.shape == gate.shape and out.dtype == gate.dtype and out.dim() == 2, "sigmoid_gate: out and gate must be [T, C] of one dtype")
+    """out *= sigmoid(gate); out [T, C] and gate [T, C], or gate [T, C / group]: one value for every `group` neighbouring columns
+    (a gate per head).  Rows may be strided (a gate that lies in a wider projection row)."""
+    _need(out.dim() == 2 and gate.dim() == 2 and out.dtype == gate.dtype and gate.shape[0] == out.shape[0] and gate.shape[1] > 0
+          and out.shape[1] % gate.shape[1] == 0, "sigmoid_gate: out [T, C] and gate [T, C / group] must be of one dtype")
     _launch("lrs_sigmoid_gate", _dev(out, "out"), _rows(out, "out"), _dev(gate, "gate"), _rows(gate, "gate"), dtype_code(out.dtype),
-            out.shape[0], out.shape[1], _stream())
+            out.shape[0], out.shape[1], out.shape[1] // gate.shape[1], _stream())
+
+
+def rotate_unit_prep(qkv: torch.Tensor, nq: int, nkv: int, d: int, dv: int, eps: float, unit: bool, cos, sin, neighbours: bool,
+                     k_pages: torch.Tensor, v_pages: torch.Tensor, slots: torch.Tensor, page_size: int) -> None:
+    """The rows of `qkv` [T, >= nq*d + nkv*d + nkv*dv] (q | k | v | whatever follows): the first 2 * cos.shape[1] dims of every q
+    and k head rotated (pairs (j, j + half), or with `neighbours` (2j, 2j + 1)), then, with `unit`, every head divided by
+    sqrt(mean of its squares + eps); q in place, k and v into the pages."""
+    tokens = qkv.shape[0]
+    stride = _rows(qkv, "qkv")
+    _need(qkv.shape[1] >= (nq + nkv) * d + nkv * dv, "rotate_unit_prep: the rows hold fewer than q, k and v")
+    rot_half = 0
+    if cos is not None:
+        rot_half = cos.shape[1]
+        _need(cos.shape[0] >= tokens and sin.shape == cos.shape and cos.is_contiguous() and sin.is_contiguous()
+              and cos.dtype == torch.float32 and sin.dtype == torch.float32, "rotate_unit_prep: rotary tables must be float32 [T, half]")
+    _need(k_pages.dim() == 4 and k_pages.shape[1:] == (nkv, page_size, d) and v_pages.shape == (k_pages.shape[0], nkv, dv, page_size),
+          f"rotate_unit_prep: key pages must be [pages, {nkv}, {page_size}, {d}] and value pages [pages, {nkv}, {dv}, {page_size}]")
+    _need(k_pages.is_contiguous() and v_pages.is_contiguous() and k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype,
+          "rotate_unit_prep: pages must be contiguous and of the activation dtype")
+    _need(slots.dtype == torch.int32 and slots.numel() >= tokens and slots.is_contiguous(), "rotate_unit_prep: slots must be int32 [T]")
+    _launch("lrs_rotate_unit_prep", _dev(qkv, "qkv"), dtype_code(qkv.dtype), tokens, stride, nq, nkv, d, dv, float(eps), int(unit),
+            None if cos is None else cos.data_ptr(), None if sin is None else sin.data_ptr(), rot_half, int(neighbours), _dev(k_pages, "k_pages"),
+            _dev(v_pages, "v_pages"), _dev(slots, "slots"), page_size, _stream())
+
+
+def gated_clamped(out: torch.Tensor, gate_up: torch.Tensor, alpha: float, limit: float) -> None:
+    """out [T, I] = g * sigmoid(alpha * g) * (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit), from gate_up [T, 2I]
+    (gate columns, then up columns)."""
+    tokens, inter = out.shape
+    _need(gate_up.shape == (tokens, 2 * inter) and gate_up.dtype == out.dtype and gate_up.is_contiguous() and out.is_contiguous(),
+          "gated_clamped: out must be [T, I] and gate_up [T, 2I], contiguous and of one dtype")
+    _need(limit > 0, "gated_clamped: the limit must be positive")
+    _launch("lrs_gated_clamped", _dev(out, "out"), _dev(gate_up, "gate_up"), dtype_code(out.dtype), tokens, inter, float(alpha), float(limit), _stream())
+
+
+def add_gathered(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor) -> None:
+    """out [T, C] float32 += table[ids[t]] (table [rows, C]; ids int32 [T] within the table)."""
+    tokens, cols = out.shape
+    _need(out.dtype == torch.float32 and out.is_contiguous() and table.dim() == 2 and table.shape[1] == cols and table.is_contiguous(),
+          "add_gathered: out must be contiguous float32 [T, C] and table contiguous [rows, C]")
+    _need(ids.dtype == torch.int32 and ids.numel() >= tokens and ids.is_contiguous(), "add_gathered: ids must be int32 [T]")
+    _launch("lrs_add_gathered", _dev(out, "out"), _dev(table, "table"), dtype_code(table.dtype), _dev(ids, "ids"), tokens, cols, _stream())
+
+
+def scale_values(x: torch.Tensor, factor: float) -> None:
+    """x *= factor over contiguous float32 values."""
+    _need(x.dtype == torch.float32 and x.is_contiguous() and x.numel() > 0, "scale_values: x must be contiguous float32")
+    _launch("lrs_scale_values", _dev(x, "x"), x.numel(), float(factor), _stream())
 
 
 def axpby(out: torch.Tensor, a: torch.Tensor, alpha: float, b: torch.Tensor, beta: float, norm_weight: torch.Tensor | None = None,
@@ -1070,7 +1135,8 @@ def decode_prepare_supported(d: int, rotates: bool) -> bool:
 def attention_decode(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                      token_request: torch.Tensor, positions: torch.Tensor, nq: int, scale: float, window: int = 0, splits: int = 1,
                      part_o: torch.Tensor | None = None, part_ml: torch.Tensor | None = None, max_context: int | None = None,
-                     prepare: "DecodePrepare | None" = None, form: int = 0, keep_first: int = 0) -> None:
+                     prepare: "DecodePrepare | None" = None, form: int = 0, keep_first: int = 0, sinks: torch.Tensor | None = None,
+                     softcap: float = 0.0) -> None:
     """attention() for a step with one query token per request, bfloat16 only; the keys of a token
     are divided between `splits` workgroups whose partial results meet in part_o / part_ml.
     keep_first (with a window and prepared heads): the first positions of a sequence stay visible behind the window; their
@@ -1113,14 +1179,15 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, 
         _dev(q, "q"), _rows(q, "q"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(block_table, "block_table"), block_table.stride(0),
         _dev(token_request, "token_request"), _dev(positions, "positions"), tokens,
         block_table.shape[1] * page_size if max_context is None else max_context, nq, nkv, d, page_size, scale, window, keep_first, splits,
-        form, *fused, _stream())
+        form, *fused, _sinks(sinks, nq, "attention_decode"), float(softcap), _stream())
 
 
 def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                       token_request: torch.Tensor, positions: torch.Tensor, qblock_token0: torch.Tensor, qblock_count: torch.Tensor,
                       nq: int, scale: float, window: int = 0, max_count: int | None = None, max_context: int | None = None,
                       splits: int = 1, part_o: torch.Tensor | None = None, part_ml: torch.Tensor | None = None,
-                      prepare: "DecodePrepare | None" = None, keep_first: int = 0) -> None:
+                      prepare: "DecodePrepare | None" = None, keep_first: int = 0, sinks: torch.Tensor | None = None,
+                      softcap: float = 0.0) -> None:
     """attention() on matrix cores for any bfloat16 step.  qblock_token0 / qblock_count list groups of at
     most attention_prefill_group() consecutive tokens of one request that together cover every token of
     the step once; `max_count` is the largest count among them (the group limit if not given) and
@@ -1169,7 +1236,8 @@ def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor,
         _dev(qblock_token0, "qblock_token0"), _dev(qblock_count, "qblock_count"), n_blocks,
         attention_prefill_group() if max_count is None else max_count,
         block_table.shape[1] * page_size if max_context is None else max_context, nq, nkv, d, page_size, scale, window, keep_first,
-        tokens, splits, None if slots == 1 else _dev(part_o, "part_o"), None if slots == 1 else _dev(part_ml, "part_ml"), *fused, _stream())
+        tokens, splits, None if slots == 1 else _dev(part_o, "part_o"), None if slots == 1 else _dev(part_ml, "part_ml"), *fused,
+        _sinks(sinks, nq, "attention_prefill"), float(softcap), _stream())
 
 
 def attention_prefill_prepares(d: int) -> bool:
@@ -1399,7 +1467,7 @@ class RouteRule:
     keep: int = 0
     scale: float = 1.0
 
-    KINDS = ("softmax_chosen", "sigmoid")
+    KINDS = ("softmax_chosen", "sigmoid", "sigmoid_scores")     # the last: chosen as under "sigmoid", weighted by the chosen s themselves (times scale)
 
     def words(self) -> tuple:
         _need(self.kind in self.KINDS, f"unknown routing rule {self.kind!r}; known: {', '.join(self.KINDS)}")
@@ -1457,41 +1525,59 @@ def moe_route_align(logits: torch.Tensor, bias: torch.Tensor | None, ids: torch.
 
 
 def moe_experts(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, sorted_pairs: torch.Tensor, tile_expert: torch.Tensor, tile: int, top: int,
-                gather: bool, relu_squared: bool, silu_pairs: bool = False) -> None:
+                gather: bool, relu_squared: bool, silu_pairs: bool = False, clamped_pairs: tuple | None = None,
+                pair_weights: torch.Tensor | None = None) -> None:
     """out [tiles * tile rows, N] = rows of `a` times w[expert of the tile] [N, K], transposed, for every tile in use.
     tile: rows of a tile, as moe_tile_rows() gave them for the step that was sorted.
     gather: the row of a sorted pair is a[pair // top] (tokens); else `a` is in sorted order itself.
-    silu_pairs: w holds a gate row 2j and an up row 2j + 1 for every feature j, and out [*, N / 2] = silu(gate) * up."""
+    silu_pairs: w holds a gate row 2j and an up row 2j + 1 for every feature j, and out [*, N / 2] = silu(gate) * up.
+    clamped_pairs (alpha, limit): the same rows, out = g * sigmoid(alpha * g) * (u + 1) with g = min(p * gate, limit) and
+    u = clamp(p * up, -limit, limit); p = pair_weights[pair] (float32 [T * top], the weight of the row's (token, choice) pair:
+    the expert runs on p times its input) or 1."""
     experts, n, k = w.shape
     tiles = tile_expert.numel()
     _need(tile in (32, 128), "moe_experts: tiles have 32 or 128 rows")
     _need(w.is_contiguous() and a.dtype == w.dtype and a.shape[1] == k, "moe_experts: a [*, K] and w [E, N, K] must agree")
-    _need(not (relu_squared and silu_pairs) and (not silu_pairs or n % 4 == 0), "moe_experts: one activation, and pairs of rows four at a time")
-    _need(out.shape == (tiles * tile, n // 2 if silu_pairs else n) and out.dtype in (w.dtype, torch.float32), "moe_experts: out must be [tiles * tile rows, N] (N / 2 for pairs)")
+    pairs_act = silu_pairs or clamped_pairs is not None
+    _need(relu_squared + silu_pairs + (clamped_pairs is not None) <= 1 and (not pairs_act or n % 4 == 0), "moe_experts: one activation, and pairs of rows four at a time")
+    _need(pair_weights is None or (clamped_pairs is not None and pair_weights.dtype == torch.float32 and pair_weights.is_contiguous()),
+          "moe_experts: weights on the inputs are float32 and come with the clamped activation")
+    alpha, limit = clamped_pairs if clamped_pairs is not None else (0.0, 0.0)
+    _need(out.shape == (tiles * tile, n // 2 if pairs_act else n) and out.dtype in (w.dtype, torch.float32), "moe_experts: out must be [tiles * tile rows, N] (N / 2 for pairs)")
     _need(gather or a.shape[0] >= tiles * tile, "moe_experts: sorted rows missing")
     _need(sorted_pairs.numel() >= tiles * tile, "moe_experts: sorted list too short")
     _launch("lrs_moe_experts", _dev(out, "out"), dtype_code(out.dtype), _rows(out, "out"), _dev(a, "a"), _dev(w, "w"), dtype_code(w.dtype),
             _rows(a, "a"), n, k, _dev(sorted_pairs, "sorted_pairs", torch.int32), _dev(tile_expert, "tile_expert", torch.int32), tiles, tile, top,
-            int(gather), 2 if silu_pairs else int(relu_squared), _stream())
+            int(gather), 3 if clamped_pairs is not None else 2 if silu_pairs else int(relu_squared),
+            None if pair_weights is None else _dev(pair_weights, "pair_weights"), float(alpha), float(limit), _stream())
 
 
-def moe_combine(residual: torch.Tensor, rows: torch.Tensor, place: torch.Tensor, weights: torch.Tensor, norm_weight: torch.Tensor | None,
-                eps: float = 0.0, rounded: torch.Tensor | None = None, layer_norm_alpha: float | None = None) -> None:
+def moe_combine(residual: torch.Tensor, rows: torch.Tensor, place: torch.Tensor, weights: torch.Tensor | None, norm_weight: torch.Tensor | None,
+                eps: float = 0.0, rounded: torch.Tensor | None = None, layer_norm_alpha: float | None = None, top: int | None = None,
+                extra: torch.Tensor | None = None) -> None:
     """residual [T, H] += sum over a token's choices of weights[t, c] * rows[place[t, c]]; with norm_weight: the RMS
     norm (weight norm_weight, eps) of that sum instead of the sum itself; with layer_norm_alpha as well: residual becomes
     the layer norm (norm_weight, eps) of layer_norm_alpha * residual + sum.  rounded: bfloat16 [T, H] that receives the
-    updated rows as well."""
-    tokens, top = weights.shape
+    updated rows as well.  weights None (then `top` says how many choices a token has): every choice counts once.  extra
+    (float32 [T, H]): rows added to a token's sum before any norm (what a part that runs for every token gave out)."""
+    if weights is not None:
+        tokens, top = weights.shape
+    else:
+        _need(top is not None and top > 0, "moe_combine: without weights the number of choices must be given")
+        tokens = place.numel() // top if extra is None else extra.shape[0]
     hidden = rows.shape[1]
     _need(residual.dtype == torch.float32 and residual.is_contiguous() and residual.shape[0] >= tokens and residual.shape[1] == hidden
           and rows.dtype == torch.float32 and rows.is_contiguous(), "moe_combine: residual [T, H] and rows [*, H] must be contiguous float32")
-    _need(place.dtype == torch.int32 and place.numel() >= tokens * top and place.is_contiguous() and weights.dtype == torch.float32
-          and weights.is_contiguous(), "moe_combine: place must be int32 [T * top] and weights float32 [T, top]")
+    _need(place.dtype == torch.int32 and place.numel() >= tokens * top and place.is_contiguous() and (weights is None or (weights.dtype == torch.float32
+          and weights.is_contiguous())), "moe_combine: place must be int32 [T * top] and weights float32 [T, top]")
+    _need(extra is None or (extra.dtype == torch.float32 and extra.is_contiguous() and extra.shape[0] >= tokens and extra.shape[1] == hidden),
+          "moe_combine: extra rows must be contiguous float32 [T, H]")
     _need(norm_weight is None or (norm_weight.numel() == hidden and norm_weight.is_contiguous()), "moe_combine: norm weight must hold H values")
     _need(layer_norm_alpha is None or norm_weight is not None, "moe_combine: a layer norm needs its weight")
-    _launch("lrs_moe_combine", _dev(residual, "residual"), _dev(rows, "rows"), tokens, hidden, _dev(place, "place"), _dev(weights, "weights"), top,
+    _launch("lrs_moe_combine", _dev(residual, "residual"), _dev(rows, "rows"), tokens, hidden, _dev(place, "place"), None if weights is None else _dev(weights, "weights"), top,
             None if norm_weight is None else _dev(norm_weight, "norm_weight"), 0 if norm_weight is None else dtype_code(norm_weight.dtype), eps,
-            _rounded(rounded, tokens, hidden, "moe_combine"), int(layer_norm_alpha is not None), 0.0 if layer_norm_alpha is None else layer_norm_alpha, _stream())
+            _rounded(rounded, tokens, hidden, "moe_combine"), int(layer_norm_alpha is not None), 0.0 if layer_norm_alpha is None else layer_norm_alpha,
+            None if extra is None else _dev(extra, "extra"), _stream())
 
 
 # ------------------------------------------------------------------- latent attention

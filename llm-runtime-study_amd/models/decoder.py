@@ -35,7 +35,7 @@ class DecoderModel:
         spec = self.spec
         out = {spec.embedding_name: TensorSpec((spec.vocab_size, spec.hidden_size), role="embedding")}
         for index, layer in enumerate(self.layers):
-            prefix = spec.layer_prefix.format(index=index)
+            prefix = spec.layer_prefix_of(index)
             out.update({f"{prefix}.{name}": t for name, t in layer.tensors().items()})
         out.update({f"{spec.final_norm_prefix}.{name}": t for name, t in self.final_norm.tensors().items()})
         for part, prefix in self._around():
@@ -55,7 +55,7 @@ class DecoderModel:
         head = weights.get(spec.head_name)
         self.head = self.embedding if head is None else head.to(dtype).contiguous()
         for index, layer in enumerate(self.layers):
-            prefix = spec.layer_prefix.format(index=index) + "."
+            prefix = spec.layer_prefix_of(index) + "."
             layer.bind(under(weights, prefix), dtype)
         for part, prefix in [(self.final_norm, spec.final_norm_prefix)] + self._around():
             prefix += "."

@@ -12,6 +12,9 @@ An architecture turns its typed configuration into a ModelSpec; everything after
             stream right after the embedding (a learned or absolute position signal, a scale)
             and on the float32 logits (a scale, a soft cap); their tensors are named
             `<after_embedding_prefix>.<name>` and `<after_head_prefix>.<name>`.
+  layer_numbers
+            the number each distinct layer's tensors carry in `layer_prefix`, where that is not its place in `layers` (a
+            checkpoint that numbers the runs of the schedule and stores the tensors of a shared layer once).
   checkpoint_name
             for checkpoints that name their tensors otherwise than the parts do: the function from a part's
             full tensor name to the checkpoint's.
@@ -53,6 +56,7 @@ class ModelSpec:
     after_head: PartSpec | None = None
     after_embedding_prefix: str = "model.after_embedding"
     after_head_prefix: str = "after_head"
+    layer_numbers: tuple[int, ...] | None = None
     # the checkpoint's name of a tensor, given the name the parts make for it (prefixes and all); None: the same
     checkpoint_name: Callable[[str], str] | None = field(default=None, compare=False)
     extra: dict = field(default_factory=dict, compare=False)
@@ -60,6 +64,8 @@ class ModelSpec:
     def validate(self) -> None:
         if not self.layers:
             raise ValueError("a model needs at least one layer")
+        if self.layer_numbers is not None and (len(self.layer_numbers) != len(self.layers) or len(set(self.layer_numbers)) != len(self.layers)):
+            raise ValueError(f"layer_numbers must give each of the {len(self.layers)} layers a number of its own")
         for position, entry in enumerate(self.schedule):
             if not 0 <= entry.layer < len(self.layers):
                 raise ValueError(f"schedule entry {position} names layer {entry.layer}, but there are {len(self.layers)} layers")
@@ -68,3 +74,7 @@ class ModelSpec:
                     raise ValueError(f"schedule entry {position} may only read the cache of an earlier entry, got {entry.cache_from}")
                 if self.schedule[entry.cache_from].cache_from is not None:
                     raise ValueError(f"schedule entry {position} reads entry {entry.cache_from}, which owns no cache itself")
+
+    def layer_prefix_of(self, index: int) -> str:
+        """The prefix of the tensors of layer `index` of `layers`."""
+        return self.layer_prefix.format(index=index if self.layer_numbers is None else self.layer_numbers[index])

@@ -22,6 +22,13 @@ keys keep their positions); `output_gate` multiplies the heads' outputs by sigmo
 gate's matrix is stacked behind q, k and v).  A layer with any of them prepares its heads with `qkv_norm_prep`; its attention
 runs on the matrix cores where the shape allows (bfloat16, values as wide as keys; the kept positions' keys are then one more
 partial result beside those of the window's splits, which the merge of the splits adds in) and in the any-shape kernel otherwise.
+
+And these, served by the same path: `unit_norm_after_rotation` divides every q and k head by its own root mean square (no
+weight, `qk_norm_eps`) after the rotation instead of a weighted norm before it (`rotate_unit_prep` prepares the heads; the
+position part says whether a pair is (i, i + rot/2) or (2i, 2i + 1)); `sink` adds a learned term exp(sink_h) per head to the
+softmax's denominator, which has no key and no value; `score_cap` passes the scaled scores through cap * tanh(score / cap);
+`output_gate="head"` gates with one number a head, sigmoid(W_g x)_h, where `True` gates every value; `bias` with any of these
+adds the stacked biases in the projection.
 """
 
 from __future__ import annotations
@@ -47,7 +54,8 @@ class GQAAttention(Part):
                  position: PartSpec = PartSpec("none"), qk_norm: bool = False, qk_norm_eps: float = 1e-6,
                  bias: bool = False, scale: float | None = None, window: int | None = None,
                  kv_shared: bool = False, values_from_keys: bool = False, norm_over: str = "head", value_dim: int | None = None,
-                 keep_first: int = 0, output_gate: bool = False):
+                 keep_first: int = 0, output_gate: bool | str = False, unit_norm_after_rotation: bool = False, sink: bool = False,
+                 score_cap: float | None = None):
         for name, value in (("hidden_size", hidden_size), ("num_heads", num_heads), ("num_kv_heads", num_kv_heads), ("head_dim", head_dim)):
             if value <= 0:
                 raise ValueError(f"{name} must be positive, got {value}")
@@ -72,12 +80,27 @@ class GQAAttention(Part):
             raise ValueError(f"value_dim must be positive when given, got {value_dim}")
         if keep_first < 0 or (keep_first and window is None):
             raise ValueError(f"keep_first must not be negative and needs a window, got {keep_first}")
+        if output_gate not in (False, True, "head"):
+            raise ValueError(f"output_gate must be False, True (a gate a value) or 'head' (a gate a head), got {output_gate!r}")
+        if score_cap is not None and (not math.isfinite(score_cap) or score_cap <= 0):
+            raise ValueError(f"score_cap must be finite and positive when given, got {score_cap}")
+        if unit_norm_after_rotation and qk_norm:
+            raise ValueError("heads are normalised before the rotation with a weight (qk_norm) or after it without one, not both")
+        if unit_norm_after_rotation and qk_norm_eps <= 0:
+            raise ValueError(f"qk_norm_eps must be positive, got {qk_norm_eps}")
         self.norm_over, self.value_dim, self.keep_first, self.output_gate = norm_over, value_dim or head_dim, keep_first, output_gate
-        # the forms that the kernel preparing whole rows serves (see the module's text)
-        self.whole_rows = (qk_norm and norm_over == "projection") or self.value_dim != head_dim or keep_first > 0 or output_gate
-        if self.whole_rows and (kv_shared or values_from_keys or bias or (qk_norm and norm_over == "head")):
-            raise ValueError("a norm over the projection, values of their own size, kept first positions and an output gate come "
-                             "without biases, shared or key-made values and per-head norms")
+        self.unit_after, self.has_sink, self.score_cap = unit_norm_after_rotation, sink, score_cap
+        self.neighbours = getattr(self.position, "pairing", "halves") == "interleaved"
+        # the forms that the kernels preparing whole rows serve (see the module's text)
+        self.whole_rows = bool((qk_norm and norm_over == "projection") or self.value_dim != head_dim or keep_first > 0 or output_gate
+                               or unit_norm_after_rotation or sink or score_cap is not None or self.neighbours)
+        if self.whole_rows and (kv_shared or values_from_keys or (qk_norm and norm_over == "head")):
+            raise ValueError("a norm over the projection or after the rotation, values of their own size, kept first positions, a sink, "
+                             "capped scores and an output gate come without shared or key-made values and per-head norms before the rotation")
+        if self.neighbours and qk_norm:
+            raise ValueError("neighbouring pairs are rotated by the kernel that normalises after the rotation or not at all")
+        self.gate_width = 0 if not output_gate else num_heads if output_gate == "head" else num_heads * self.value_dim
+        self.sinks = None
         self.w_qkv = self.b_qkv = self.w_o = self.q_norm = self.k_norm = None
 
     # ------------------------------------------------------------------ weights
@@ -89,7 +112,9 @@ class GQAAttention(Part):
         if self.bias:
             specs.update({f"{n}.bias": TensorSpec((widths[n],), role="bias") for n in names})
         if self.output_gate:
-            specs["g_proj.weight"] = TensorSpec((self.num_heads * self.value_dim, h))
+            specs["g_proj.weight"] = TensorSpec((self.gate_width, h))
+        if self.has_sink:
+            specs["sink"] = TensorSpec((self.num_heads,), role="bias")
         specs["o_proj.weight"] = TensorSpec((h, self.num_heads * self.value_dim))
         if self.qk_norm:
             over = d if self.norm_over == "head" else None
@@ -102,8 +127,17 @@ class GQAAttention(Part):
         names = ("q_proj",) if self.kv_shared else ("q_proj", "k_proj", "k_proj") if self.values_from_keys else ("q_proj", "k_proj", "v_proj")
         if self.output_gate:
             names += ("g_proj",)
-        self.w_qkv = torch.cat([weights[f"{n}.weight"] for n in names], 0).to(dtype).contiguous()
-        self.b_qkv = torch.cat([weights[f"{n}.bias"] for n in names], 0).to(dtype).contiguous() if self.bias else None
+        stacked = [weights[f"{n}.weight"] for n in names]
+        biases = [weights[f"{n}.bias"] if n != "g_proj" else weights["g_proj.weight"].new_zeros(self.gate_width) for n in names] if self.bias else None
+        pad = -sum(w.shape[0] for w in stacked) % 16 if self.whole_rows else 0     # rows of whole groups of 16 columns suit every product kernel
+        if pad:
+            stacked.append(stacked[0].new_zeros(pad, self.hidden_size))
+            if biases is not None:
+                biases.append(biases[0].new_zeros(pad))
+        self.w_qkv = torch.cat(stacked, 0).to(dtype).contiguous()
+        self.b_qkv = torch.cat(biases, 0).to(dtype).contiguous() if self.bias else None
+        if self.has_sink:
+            self.sinks = weights["sink"].float().contiguous()
         self.w_o = weights["o_proj.weight"].to(dtype).contiguous()
         if self.qk_norm:
             self.q_norm = weights["q_norm.weight"]
@@ -297,9 +331,14 @@ class GQAAttention(Part):
         t, d, dv, nq, nkv = rows_of(x), self.head_dim, self.value_dim, self.num_heads, self.num_kv_heads
         gate_at = (nq + nkv) * d + nkv * dv
         qkv = ctx.scratch("attn_qkvg", (t, self.w_qkv.shape[0]), ctx.dtype)
-        linear(ctx, qkv, x, self.w_qkv)
-        ops.qkv_norm_prep(qkv, nq, nkv, d, dv, self.q_norm, self.k_norm, self.qk_norm_eps, cos, sin, cache.k_pages, cache.v_pages,
-                          group.slots, group.page_size)
+        linear(ctx, qkv, x, self.w_qkv, self.b_qkv)
+        if self.unit_after or self.neighbours:
+            ops.rotate_unit_prep(qkv, nq, nkv, d, dv, self.qk_norm_eps, self.unit_after, cos, sin, self.neighbours, cache.k_pages, cache.v_pages,
+                                 group.slots, group.page_size)
+        else:
+            ops.qkv_norm_prep(qkv, nq, nkv, d, dv, self.q_norm, self.k_norm, self.qk_norm_eps, cos, sin, cache.k_pages, cache.v_pages,
+                              group.slots, group.page_size)
+        more = {"sinks": self.sinks, "softcap": self.score_cap or 0.0}
         out = ctx.scratch("attn_out", (t, nq * dv), ctx.dtype)
         cores = dv == d and ops.attention_decode_supported(ctx.dtype, nq, nkv, d, group.page_size)
         extra = 1 if self.keep_first else 0      # the kept first positions' share is one more partial result for the merge
@@ -314,7 +353,7 @@ class GQAAttention(Part):
                 part_ml = ctx.scratch("attn_part_ml", (t, nq * (splits + extra) * 2), torch.float32)
             ops.attention_decode(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_slot, ctx.positions,
                                  nq, self.scale, self.window or 0, splits, part_o, part_ml, ctx.max_k_bound, None, form=1,
-                                 keep_first=self.keep_first)
+                                 keep_first=self.keep_first, **more)
         elif cores:
             longest = ctx.max_k_bound if self.window is None else min(ctx.max_k_bound, self.window + 64)
             singles = ctx.single_rows
@@ -326,7 +365,7 @@ class GQAAttention(Part):
                     part_ml = ctx.scratch("attn_single_part_ml", (singles, nq * (splits + extra) * 2), torch.float32)
                 ops.attention_decode(out[:singles], qkv[:singles], cache.k_pages, cache.v_pages, group.block_table, ctx.token_slot,
                                      ctx.positions, nq, self.scale, self.window or 0, splits, part_o, part_ml, ctx.max_k_bound, None, form=1,
-                                     keep_first=self.keep_first)
+                                     keep_first=self.keep_first, **more)
             rest = ctx.memo.get("rows_after_singles")
             if rest is None:
                 rest = ctx.memo["rows_after_singles"] = (ctx.token_slot[singles:], ctx.positions[singles:])
@@ -337,12 +376,12 @@ class GQAAttention(Part):
                 part_ml = ctx.scratch("attn_part_ml", (t - singles, nq * (splits + extra) * 2), torch.float32)
             ops.attention_prefill(out[singles:], qkv[singles:], cache.k_pages, cache.v_pages, group.block_table, rest[0], rest[1],
                                   ctx.qblock_token0, ctx.qblock_count, nq, self.scale, self.window or 0, ctx.max_qblock, ctx.max_k_bound,
-                                  splits, part_o, part_ml, None, keep_first=self.keep_first)
+                                  splits, part_o, part_ml, None, keep_first=self.keep_first, **more)
         else:
             ops.attention(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_slot, ctx.positions, nq, self.scale,
-                          self.window or 0, self.keep_first)
+                          self.window or 0, self.keep_first, **more)
         if self.output_gate:
-            ops.sigmoid_gate(out, qkv[:, gate_at:gate_at + nq * dv])
+            ops.sigmoid_gate(out, qkv[:, gate_at:gate_at + self.gate_width])
         return linear(ctx, residual, out, self.w_o, accumulate=accumulate, then_norm=then_norm)
 
 

@@ -1,4 +1,5 @@
-"""Feed-forwards.  SwiGLU: down(silu(gate(x)) * up(x)), three bias-free projections; DenseMLP (at the end of the file):
+"""Feed-forwards.  SwiGLU: down(silu(gate(x)) * up(x)), three bias-free projections (with `activation="clamped"` the gated
+activation is g * sigmoid(alpha g) * (u + 1), g = min(gate(x), limit), u = clamp(up(x), -limit, limit)); DenseMLP (at the end of the file):
 down(act(up(x))), two bias-free projections with an activation between them.
 
 Reference mini_llm/nn/mlp.py:80-87.  gate and up are stacked into one [2I, H] matrix when
@@ -22,10 +23,16 @@ class SwiGLU(Part):
     begins_next_norm = True
     can_overwrite = True        # forward(..., accumulate=False) stores its output
 
-    def __init__(self, hidden_size: int, intermediate_size: int):
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu", alpha: float = 1.702, limit: float | None = None):
         if hidden_size <= 0 or intermediate_size <= 0:
             raise ValueError("hidden_size and intermediate_size must be positive")
+        if activation not in ("silu", "clamped"):
+            raise ValueError(f"unknown gated activation {activation!r}; known: silu, clamped")
+        if activation == "clamped" and (limit is None or not limit > 0):
+            raise ValueError(f"the clamped activation needs a positive limit, got {limit}")
         self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
+        # "clamped": down(g * sigmoid(alpha g) * (u + 1)) with g = min(gate(x), limit), u = clamp(up(x), -limit, limit)
+        self.clamped = None if activation == "silu" else (float(alpha), float(limit))
         self.gate_up = self.down = None
 
     def tensors(self):
@@ -42,7 +49,7 @@ class SwiGLU(Part):
         # bfloat16: rows interleaved in groups of 8 (8 gate rows, then the 8 up rows of the same
         # features), so that the product's epilogue has both halves of a feature and writes
         # silu(gate) * up itself; otherwise gate rows then up rows and a separate activation kernel
-        self.interleaved = dtype == torch.bfloat16 and i % 8 == 0 and h % 8 == 0
+        self.interleaved = dtype == torch.bfloat16 and i % 8 == 0 and h % 8 == 0 and self.clamped is None
         if self.interleaved:
             self.gate_up = torch.stack((gate.view(i // 8, 8, h), up.view(i // 8, 8, h)), 1).reshape(2 * i, h).contiguous()
         else:
@@ -60,7 +67,10 @@ class SwiGLU(Part):
         else:
             gate_up = ctx.scratch("ffn_gate_up", (t, 2 * self.intermediate_size), ctx.dtype)
             linear(ctx, gate_up, x, self.gate_up)
-            ops.silu_mul(act, gate_up)
+            if self.clamped is not None:
+                ops.gated_clamped(act, gate_up, *self.clamped)
+            else:
+                ops.silu_mul(act, gate_up)
         return linear(ctx, residual, act, self.down, accumulate=accumulate, then_norm=then_norm)
 
 

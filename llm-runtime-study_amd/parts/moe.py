@@ -5,8 +5,11 @@
     rule "sigmoid":         s = sigmoid(z); chosen = the `top` largest s + bias (the bias takes part in the choice only;
                             with groups, among the experts of the `keep` groups whose two largest s + bias sum highest);
                             p = s[chosen] / (sum of s[chosen] + 1e-20) * scale
-    out = sum over chosen e of p_e * expert_e(x)
+    rule "sigmoid_scores":  chosen as under "sigmoid"; p = s[chosen] * scale (the scores as they are, not divided by their sum)
+    out = sum over chosen e of p_e * expert_e(x), or with `weight_on="input"` the sum of expert_e(p_e * x)
     expert "relu_squared":  W_down relu(W_up x)^2;   "silu_gated":  W_down (silu(W_gate x) * (W_up x))
+    expert "clamped_gated": W_down (g * sigmoid(alpha g) * (u + 1)) with g = min(W_gate x, limit), u = clamp(W_up x, -limit, limit)
+    `shared`: a feed-forward part that runs for every token; its output is added to the experts' sum (before a layer's norm).
 
 On the device: the router product, the choice per token, one sort of the step's (token, choice) pairs by expert
 into runs padded to whole row tiles, two grouped products over the sorted rows (the activation in the first one's
@@ -21,22 +24,21 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import Part, TensorSpec, register
+from .base import Part, PartSpec, TensorSpec, create, flops_of, register, under
 from .linear import kernels_of, materialize, rows_of, workspace_of
 
-ACTIVATIONS = ("relu_squared", "silu_gated")
+ACTIVATIONS = ("relu_squared", "silu_gated", "clamped_gated")
 
 
 class RoutedExperts(Part):
-    graph_safe = True
-    plan_safe = True
     applies_output_norm = True    # forward(..., output_norm=norm): residual += norm(out) instead of residual += out
     applies_sum_norm = True       # forward(..., sum_norm=(norm, alpha)): residual = norm(alpha * residual + out), for a layer norm
     rounds_stream = True          # forward(..., rounded=buffer): the updated stream is left there in bfloat16 as well
 
     def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, top: int, router_bias: bool = False,
                  activation: str = "relu_squared", rule: str = "softmax_chosen", groups: int = 0, keep: int = 0, weight_scale: float = 1.0,
-                 bias_name: str = "router.bias"):
+                 bias_name: str = "router.bias", weight_on: str = "output", activation_alpha: float = 1.702, activation_limit: float | None = None,
+                 shared: PartSpec | None = None):
         if min(hidden_size, intermediate_size, num_experts, top) <= 0:
             raise ValueError("hidden_size, intermediate_size, num_experts and top must be positive")
         if top > num_experts:
@@ -54,8 +56,29 @@ class RoutedExperts(Part):
             raise ValueError(f"{num_experts} experts in {groups} groups of which {keep} are kept cannot give {top} choices under rule {rule!r}")
         if not weight_scale > 0:
             raise ValueError(f"weight_scale must be positive, got {weight_scale}")
-        self.gated = activation == "silu_gated"
+        self.gated = activation in ("silu_gated", "clamped_gated")
+        self.clamped = None
+        if activation == "clamped_gated":
+            if activation_limit is None or not activation_limit > 0:
+                raise ValueError(f"the clamped activation needs a positive limit, got {activation_limit}")
+            self.clamped = (float(activation_alpha), float(activation_limit))
+        if weight_on not in ("output", "input"):
+            raise ValueError(f"weight_on must be 'output' or 'input', got {weight_on!r}")
+        if weight_on == "input" and self.clamped is None:
+            raise ValueError("weights on the experts' inputs are served by the clamped gated activation's kernels only")
+        self.weight_on = weight_on
+        self.shared = None if shared is None else create("feed_forward", shared)
+        if self.shared is not None and not getattr(self.shared, "can_overwrite", False):
+            raise ValueError("a shared expert must be able to store its output (can_overwrite)")
         self.router = self.bias = self.up = self.down = None
+
+    @property
+    def graph_safe(self) -> bool:
+        return self.shared is None or getattr(self.shared, "graph_safe", False)
+
+    @property
+    def plan_safe(self) -> bool:
+        return self.shared is None or getattr(self.shared, "plan_safe", False)
 
     def tensors(self):
         h, i = self.hidden_size, self.intermediate_size
@@ -67,6 +90,8 @@ class RoutedExperts(Part):
                 specs[f"experts.{e}.gate.weight"] = TensorSpec((i, h))
             specs[f"experts.{e}.up.weight"] = TensorSpec((i, h))
             specs[f"experts.{e}.down.weight"] = TensorSpec((h, i))
+        if self.shared is not None:
+            specs.update({f"shared.{name}": spec for name, spec in self.shared.tensors().items()})
         return specs
 
     def bind(self, weights, dtype):
@@ -84,14 +109,17 @@ class RoutedExperts(Part):
         else:
             self.up = torch.stack([weights[f"experts.{e}.up.weight"].to(dtype) for e in range(self.num_experts)]).contiguous()
         self.down = torch.stack([weights[f"experts.{e}.down.weight"].to(dtype) for e in range(self.num_experts)]).contiguous()
+        if self.shared is not None:
+            self.shared.bind(under(weights, "shared."), dtype)
 
     def weight_bytes(self):
         """What a decode step of one token reads: the router and the chosen experts."""
         chosen = (3 if self.gated else 2) * self.top * self.hidden_size * self.intermediate_size
-        return (self.router.numel() + chosen) * self.up.element_size()
+        return (self.router.numel() + chosen) * self.up.element_size() + (0 if self.shared is None else self.shared.weight_bytes())
 
     def flops(self, tokens, pairs):
-        return 2.0 * tokens * (self.num_experts * self.hidden_size + (3 if self.gated else 2) * self.top * self.hidden_size * self.intermediate_size)
+        own = 2.0 * tokens * (self.num_experts * self.hidden_size + (3 if self.gated else 2) * self.top * self.hidden_size * self.intermediate_size)
+        return own + (0.0 if self.shared is None else flops_of(self.shared, tokens, pairs))
 
     def forward(self, ctx, x, residual, then_norm=None, output_norm=None, rounded=None, sum_norm=None):
         t = rows_of(x)
@@ -112,7 +140,13 @@ class RoutedExperts(Part):
             ops.moe_route(logits[:, :experts], self.bias, ids, weights, rule=self.rule)
             ops.moe_align(ids, experts, sorted_pairs, place, tile_expert)
         hidden = ctx.scratch("moe_hidden", (rows, self.intermediate_size), ctx.dtype)
-        if self.gated and self.paired:
+        on_input = self.weight_on == "input"
+        if self.clamped is not None and self.paired:
+            ops.moe_experts(hidden, x, self.up, sorted_pairs, tile_expert, tile, top, gather=True, relu_squared=False, clamped_pairs=self.clamped,
+                            pair_weights=weights if on_input else None)
+        elif self.clamped is not None:
+            raise ValueError("the clamped gated activation is made in the grouped product's epilogue, which takes an even expert size")
+        elif self.gated and self.paired:
             ops.moe_experts(hidden, x, self.up, sorted_pairs, tile_expert, tile, top, gather=True, relu_squared=False, silu_pairs=True)
         elif self.gated:    # an odd size: gate rows then up rows, and the activation as a kernel of its own
             both = ctx.scratch("moe_gate_up", (rows, 2 * self.intermediate_size), ctx.dtype)
@@ -122,14 +156,21 @@ class RoutedExperts(Part):
             ops.moe_experts(hidden, x, self.up, sorted_pairs, tile_expert, tile, top, gather=True, relu_squared=True)
         outputs = ctx.scratch("moe_outputs", (rows, self.hidden_size), torch.float32)
         ops.moe_experts(outputs, hidden, self.down, sorted_pairs, tile_expert, tile, top, gather=False, relu_squared=False)
+        extra = None
+        if self.shared is not None:      # runs for every token; its rows join the experts' sum before any norm
+            extra = ctx.scratch("moe_shared_out", (t, self.hidden_size), torch.float32)
+            self.shared.forward(ctx, x, extra, accumulate=False)
+        more = {"top": top, "extra": extra}
+        if on_input:                     # the weights went into the experts with their inputs: every choice counts once
+            weights = None
         if sum_norm is not None:
             weight, eps = sum_norm[0].layer_parameters()
-            ops.moe_combine(residual[:t], outputs, place, weights, weight, eps, rounded=rounded, layer_norm_alpha=sum_norm[1])
+            ops.moe_combine(residual[:t], outputs, place, weights, weight, eps, rounded=rounded, layer_norm_alpha=sum_norm[1], **more)
         elif output_norm is None:
-            ops.moe_combine(residual[:t], outputs, place, weights, None, rounded=rounded)
+            ops.moe_combine(residual[:t], outputs, place, weights, None, rounded=rounded, **more)
         else:
             weight, eps = output_norm.rms_parameters()
-            ops.moe_combine(residual[:t], outputs, place, weights, weight, eps, rounded=rounded)
+            ops.moe_combine(residual[:t], outputs, place, weights, weight, eps, rounded=rounded, **more)
         return None
 
 
