@@ -60,8 +60,6 @@ class FelosunExperts:
                    _positive(router, "top", where), shared_ff, shared_limit)
         if made.top > made.experts:
             raise ConfigError(f"{where}: top {made.top} exceeds the {made.experts} experts")
-        if made.ff % 2:
-            raise ConfigError(f"{where}: the experts' gated activation is made for pairs of rows, so expert.ff must be even, got {made.ff}")
         return made
 
     def to_json_dict(self) -> dict:

@@ -107,8 +107,11 @@ __device__ __forceinline__ void route_token_sigmoid(const float* __restrict__ lo
 #pragma unroll
   for (int c = 0; c < ROUTE_MAX_PER_LANE; ++c) {
     const int e = lane + WAVE * c;
-    s[c] = e < experts ? 1.0f / (1.0f + expf(-logits[(int64_t)t * ld + e])) : 0.f;
-    v[c] = e < experts ? s[c] + (bias ? bias[e] : 0.f) : -INFINITY;
+    const float z = e < experts ? logits[(int64_t)t * ld + e] : 0.f;
+    s[c] = e < experts ? 1.0f / (1.0f + expf(-z)) : 0.f;
+    // without a bias and without groups the order of the scores is the order of the logits, which does not run out of
+    // digits where the sigmoid nears one (logits of 17 and of 30 both give 1.0f)
+    v[c] = e < experts ? (bias || rule.groups > 0 ? s[c] + (bias ? bias[e] : 0.f) : z) : -INFINITY;
   }
   if (rule.groups > 0 && rule.keep < rule.groups) {
     const int per = experts / rule.groups;

@@ -48,6 +48,7 @@ class RoutedExperts(Part):
         if activation not in ACTIVATIONS:
             raise ValueError(f"unknown activation {activation!r}; known: {', '.join(ACTIVATIONS)}")
         self.hidden_size, self.intermediate_size, self.num_experts, self.top = hidden_size, intermediate_size, num_experts, top
+        self.inner = intermediate_size       # features a grouped product makes per expert (one more where an odd size is padded)
         self.router_bias, self.activation, self.bias_name = router_bias, activation, bias_name
         self.rule = ops.RouteRule(rule, groups, keep, weight_scale)
         if rule not in ops.RouteRule.KINDS:
@@ -101,6 +102,10 @@ class RoutedExperts(Part):
             router = torch.cat((router, router.new_zeros(pad, self.hidden_size)), 0)
         self.router = router.contiguous()
         self.bias = weights[self.bias_name].float().contiguous() if self.router_bias else None
+        if self.clamped is not None and self.intermediate_size % 2:
+            # an odd size: one more feature whose gate, up and down weights are zero; it gives g = u = 0, so 0 * sigmoid(0) * 1 = 0
+            self._bind_padded(weights, dtype)
+            return
         if self.gated:      # a feature's gate row, then its up row: one product makes both, and its epilogue the gated activation
             self.paired = self.intermediate_size % 2 == 0
             join = (lambda g, u: torch.stack((g, u), 1).reshape(2 * self.intermediate_size, self.hidden_size)) if self.paired else (lambda g, u: torch.cat((g, u), 0))
@@ -109,6 +114,21 @@ class RoutedExperts(Part):
         else:
             self.up = torch.stack([weights[f"experts.{e}.up.weight"].to(dtype) for e in range(self.num_experts)]).contiguous()
         self.down = torch.stack([weights[f"experts.{e}.down.weight"].to(dtype) for e in range(self.num_experts)]).contiguous()
+        if self.shared is not None:
+            self.shared.bind(under(weights, "shared."), dtype)
+
+    def _bind_padded(self, weights, dtype):
+        h, i = self.hidden_size, self.intermediate_size
+        self.paired = True
+        rows = []
+        for e in range(self.num_experts):
+            gate, up = weights[f"experts.{e}.gate.weight"].to(dtype), weights[f"experts.{e}.up.weight"].to(dtype)
+            zero = gate.new_zeros(1, h)
+            rows.append(torch.stack((torch.cat((gate, zero), 0), torch.cat((up, zero), 0)), 1).reshape(2 * (i + 1), h))
+        self.up = torch.stack(rows).contiguous()
+        self.down = torch.stack([torch.cat((weights[f"experts.{e}.down.weight"].to(dtype), self.up.new_zeros(h, 1)), 1)
+                                 for e in range(self.num_experts)]).contiguous()
+        self.inner = i + 1
         if self.shared is not None:
             self.shared.bind(under(weights, "shared."), dtype)
 
@@ -139,7 +159,7 @@ class RoutedExperts(Part):
         else:
             ops.moe_route(logits[:, :experts], self.bias, ids, weights, rule=self.rule)
             ops.moe_align(ids, experts, sorted_pairs, place, tile_expert)
-        hidden = ctx.scratch("moe_hidden", (rows, self.intermediate_size), ctx.dtype)
+        hidden = ctx.scratch("moe_hidden", (rows, self.inner), ctx.dtype)
         on_input = self.weight_on == "input"
         if self.clamped is not None and self.paired:
             ops.moe_experts(hidden, x, self.up, sorted_pairs, tile_expert, tile, top, gather=True, relu_squared=False, clamped_pairs=self.clamped,

@@ -129,8 +129,9 @@ def test_parts_refuse_what_their_kernels_do_not_take():
         create("mixer", PartSpec("gqa_attention", dict(base, keep_first=2)))
     with pytest.raises(ValueError, match="norm_over"):
         create("mixer", PartSpec("gqa_attention", dict(base, norm_over="token")))
-    with pytest.raises(ValueError, match="without biases"):
-        create("mixer", PartSpec("gqa_attention", dict(base, bias=True)))
+    with pytest.raises(ValueError, match="per-head norms"):
+        create("mixer", PartSpec("gqa_attention", dict(base, norm_over="head", keep_first=2, window=4)))
+    assert "k_proj.bias" in create("mixer", PartSpec("gqa_attention", dict(base, bias=True))).tensors()      # biases are added in the projection
     ssm = {"hidden_size": 8, "num_heads": 4, "num_groups": 2, "state_size": 8, "value_dim": 6, "conv_taps": 2, "norm_parts": 3, "norm_eps": 1e-6}
     create("mixer", PartSpec("state_space", ssm))
     with pytest.raises(ValueError, match="parts"):
