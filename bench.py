@@ -4,6 +4,7 @@
     python bench.py --design nobodra [--shape 8b] [--layers 8] ...     # the Nobodra design at the shape's layer sizes, beside the shape itself
     python bench.py --design napizen [--shape 8b] [--layers 8] ...     # the same for the Napizen design
     python bench.py --design kaposun [--shape 8b] [--layers 8] ...     # the same for the Kaposun design
+    python bench.py --design felosun [--shape 8b] [--layers 8] ...     # the Felosun design beside a Nobodra model of attention layers and experts of equal sizes
 
 A step is one decode step of the whole engine (scheduler, step function, sampling) at the
 given batch; `value` is decoded tokens per second.  The same line carries the prefill rate
@@ -28,7 +29,7 @@ if str(ROOT) not in sys.path:
 HBM_PEAK = 8.0e12
 FLOP_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
 
-from llm_runtime_study_amd.benchmarks.shapes import QWEN3_8B, SHAPES, kaposun_like, napizen_like, nobodra_like  # noqa: E402  (layer sizes of the 8B, 14B and 32B models)
+from llm_runtime_study_amd.benchmarks.shapes import QWEN3_8B, SHAPES, felosun_like, kaposun_like, napizen_like, nobodra_like  # noqa: E402  (layer sizes of the 8B, 14B and 32B models)
 
 FULL_LAYERS = QWEN3_8B["num_hidden_layers"]
 BENCHMARK_CONTEXT = 4096      # tokens a request's cache can hold at the least: the benchmark context of the 8B configuration
@@ -48,7 +49,7 @@ def parse_args():
     parser.add_argument("--num-pages", type=int, default=None, help="pages of the cache pool (default: max-seq-len tokens for every request of the largest batch)")
     parser.add_argument("--shape", choices=tuple(SHAPES), default="8b", help="layer sizes: Qwen3-8B (default), 14B or 32B")
     parser.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (reported in config)")
-    parser.add_argument("--design", choices=("qwen3", "nobodra", "napizen", "kaposun"), default="qwen3",
+    parser.add_argument("--design", choices=("qwen3", "nobodra", "napizen", "kaposun", "felosun"), default="qwen3",
                         help="nobodra, napizen, kaposun: measure that design at the shape's layer sizes (8 layers unless --layers says otherwise) and, beside it, the shape itself with as many layers")
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
@@ -240,7 +241,7 @@ def measure_design(args, config, dtype_name: str, max_seq_len: int, max_batch: i
 
 
 def design_main(args) -> int:
-    """--design nobodra | napizen | kaposun: the design at the shape's layer sizes, and the shape itself with as many layers, one after the other."""
+    """--design nobodra | napizen | kaposun | felosun: the design at the shape's layer sizes, and the shape itself with as many layers, one after the other."""
     import gc
 
     import torch
@@ -252,12 +253,16 @@ def design_main(args) -> int:
     max_batch = args.batch if args.no_points else max(args.batch, 64)
     max_seq_len = args.max_seq_len or max(BENCHMARK_CONTEXT, args.context + args.steps + warmup_room(args.warmup, max(args.decode_steps_per_launch, 1))
                                           + decode_lead(max_batch, args.context, max(2048, args.prefill_tokens)) + max_batch + 64, args.prefill_tokens + 1)
-    name = {"nobodra": "Nobodra", "napizen": "Napizen", "kaposun": "Kaposun"}[args.design]
-    raw = {"nobodra": nobodra_like, "napizen": napizen_like, "kaposun": kaposun_like}[args.design](SHAPES[args.shape], layers)
+    name = {"nobodra": "Nobodra", "napizen": "Napizen", "kaposun": "Kaposun", "felosun": "Felosun"}[args.design]
+    raw = {"nobodra": nobodra_like, "napizen": napizen_like, "kaposun": kaposun_like, "felosun": felosun_like}[args.design](SHAPES[args.shape], layers)
     mine = measure_design(args, config_from_dict(raw), dtype_name, max_seq_len, max_batch)
     gc.collect()
     torch.cuda.empty_cache()
-    beside = measure_design(args, config_from_dict(dict(SHAPES[args.shape], num_hidden_layers=layers)), dtype_name, max_seq_len, max_batch)
+    # Felosun stands beside the model nearest to it: Nobodra's layers of windowed attention and routed experts (the same block that
+    # normalises outputs), at equal sizes; the others beside the dense shape itself
+    beside_raw = nobodra_like(SHAPES[args.shape], layers, attention_only=True) if args.design == "felosun" else dict(SHAPES[args.shape], num_hidden_layers=layers)
+    beside_name = "Nobodra, attention layers only, at the same sizes" if args.design == "felosun" else f"Qwen3-{args.shape.upper()} shape"
+    beside = measure_design(args, config_from_dict(beside_raw), dtype_name, max_seq_len, max_batch)
     main_point = mine[f"decode_b{args.batch}"]
     line = {
         "metric": f"decode tok/s at batch {args.batch} ({name} at Qwen3-{args.shape.upper()} layer sizes, {layers} layers)",
@@ -270,7 +275,7 @@ def design_main(args) -> int:
                    "mlp": [raw["layers"][0]["mlp"], raw["layers"][-1]["mlp"]],
                    "global_batch": args.batch, "seq_len": args.context, "max_seq_len": max_seq_len, "prefill_tokens": args.prefill_tokens, "parallelism": "single GPU"},
         args.design: mine,
-        "beside": {"model": f"Qwen3-{args.shape.upper()} shape, {layers} layers", **beside},
+        "beside": {"model": f"{beside_name}, {layers} layers", **beside},
     }
     print(json.dumps(line))
     return 0

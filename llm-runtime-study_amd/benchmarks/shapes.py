@@ -18,9 +18,10 @@ SHAPES = {
 }
 
 
-def nobodra_like(shape: dict, layers: int, experts: int = 32, top: int = 8, window: int = 4096) -> dict:
+def nobodra_like(shape: dict, layers: int, experts: int = 32, top: int = 8, window: int = 4096, attention_only: bool = False) -> dict:
     """A Nobodra configuration with the layer sizes of a dense shape above, for measurements beside it: the same width,
-    vocabulary and heads; three gated-delta-rule layers to every sliding-window attention layer; the dense feed-forward's
+    vocabulary and heads; three gated-delta-rule layers to every sliding-window attention layer (with `attention_only` every
+    layer is a sliding-window attention layer); the dense feed-forward's
     three matrices of `intermediate_size` as `top` of `experts` experts of two matrices each with as many weights in use
     per token (to a multiple of 128); half of every attention head rotated."""
     width, heads, kv_heads, dim = shape["hidden_size"], shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"]
@@ -30,7 +31,23 @@ def nobodra_like(shape: dict, layers: int, experts: int = 32, top: int = 8, wind
                                                             "mask": {"size": window}, "rot": {"base": 1000000.0, "dims": dim // 2}}}
     delta = {"type": "delta", "mlp": mlp, "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "conv": 4}}
     return {"architecture": "Nobodra", "vocab": shape["vocab_size"], "width": width, "norm": {"eps": 1e-6},
-            "layers": [attention if index % 4 == 3 else delta for index in range(layers)]}
+            "layers": [attention if index % 4 == 3 or attention_only else delta for index in range(layers)]}
+
+
+def felosun_like(shape: dict, layers: int, experts: int = 32, top: int = 8, window: int = 4096, keep_first: int = 8, positions: int = 40960) -> dict:
+    """A Felosun configuration with the layer sizes of a dense shape above, for measurements beside a model of equal sizes: the
+    same width, vocabulary and heads; in turn a layer of capped attention over the whole context (half of every head rotated,
+    stretched positions, a gate a head) and a layer of windowed attention with kept first positions and sinks (half of every head
+    rotated in neighbouring pairs); `top` of `experts` clamped gated experts and a shared expert of the same size, together as
+    many weights in use per token as the dense feed-forward (to a multiple of 128)."""
+    width, heads, kv_heads, dim = shape["hidden_size"], shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"]
+    ff = max(128, round(shape["intermediate_size"] / (top + 1) / 128) * 128)
+    mlp = {"kind": "moe", "expert": {"ff": ff, "limit": 7.0}, "router": {"experts": experts, "top": top}, "shared": {"ff": ff, "limit": 7.0}}
+    sizes = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5}
+    capped = {"type": "attention_2", "mlp": mlp, "mixer": dict(sizes, rot={"base": 1000000.0, "dims": dim // 2, "scaling": {"factor": 4.0}}, softcap=50.0)}
+    windowed = {"type": "attention", "mlp": mlp, "mixer": dict(sizes, rot={"base": 10000.0, "dims": dim // 2}, mask={"size": window, "keep_first": keep_first})}
+    return {"architecture": "Felosun", "vocab": shape["vocab_size"], "width": width, "max_positions": positions, "norm": {"eps": 1e-6},
+            "embedding": {"scale": 1.0}, "logit_scale": 0.5, "layers": [(capped, windowed)[index % 2] for index in range(layers)]}
 
 
 def napizen_like(shape: dict, layers: int, experts: int = 32, top: int = 8, rank: int = 512, rot: int = 64) -> dict:

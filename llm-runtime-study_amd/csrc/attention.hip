@@ -22,12 +22,13 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 constexpr float RESCALE_STEP = 8.0f;
 
 // A cap on the scores: cap * tanh(x / cap), close to x for small |x| and within (-cap, cap) for all.  tanh by one
-// exponential, exact to a few units in the last place of float32 over the whole range.
+// exponential and one reciprocal (the hardware's, a unit in the last place each): the bfloat16 kernels' form; the kernel for
+// any shape, which also serves float32 runs, calls tanhf.
 __device__ __forceinline__ float capped(float x, float cap) {
-  const float t = x / cap;
-  const float e = __expf(-2.f * fabsf(t));
-  const float r = (1.f - e) / (1.f + e);
-  return cap * (t < 0.f ? -r : r);
+  const float t = x * __builtin_amdgcn_rcpf(cap);
+  const float e = fast_exp2(-2.f * 1.4426950408889634f * fabsf(t));       // e^(-2|t|), in (0, 1]
+  const float r = (1.f - e) * __builtin_amdgcn_rcpf(1.f + e);
+  return copysignf(cap * r, t);
 }
 
 // A sink: one more term exp(sink) in a softmax's denominator that has no key and no value.  Given sums that were taken
@@ -1134,7 +1135,8 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
 // The wave that fetched a tile waits for its own fetches (vmcnt) before the barrier that opens the
 // tile to the others; the fetches of the tile after it stay in flight.  The fetches are written in
 // assembly because the compiler would wait for all of them before any LDS read it cannot tell apart.
-template <int QB, bool MANY_WAVES, bool IDLE_WAVES>
+// CAPPED: the scaled scores pass softcap * tanh(score / softcap) (an instance of its own, so that the others keep their registers).
+template <int QB, bool MANY_WAVES, bool IDLE_WAVES, bool CAPPED>
 __global__ __launch_bounds__(MANY_WAVES ? 512 : 256, MANY_WAVES ? 1 : 2) void attention_prefill_d128_bf16_kernel(
     bf16* __restrict__ out, int out_stride, const bf16* __restrict__ q, int q_stride,
     const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
@@ -1142,7 +1144,7 @@ __global__ __launch_bounds__(MANY_WAVES ? 512 : 256, MANY_WAVES ? 1 : 2) void at
     const int* __restrict__ positions, const int* __restrict__ qblock_token0,
     const int* __restrict__ qblock_count, int n_blocks, int chunk, int nq, int nkv, int page_size, float scale,
     int window, int splits, int slots, float* __restrict__ part_o, float* __restrict__ part_ml, int prepare_q, DecodePrep prep,
-    const float* __restrict__ sinks) {
+    const float* __restrict__ sinks, float softcap) {
   constexpr int D = 128, DS = D / 32, DB = D / 16, STAGES = 3;
   constexpr int KBLOCK = 1024 + 32, KBYTES = 8 * KBLOCK, VHALF = 16 * D * 2 + 16, VBYTES = 2 * VHALF;
   constexpr int VSTAGE = (VBYTES + 63) / 64 * 64;
@@ -1274,6 +1276,16 @@ __global__ __launch_bounds__(MANY_WAVES ? 512 : 256, MANY_WAVES ? 1 : 2) void at
       for (int e = 0; e < DB; ++e) o[b][e] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
 
+    // the cap, in units of the unscaled scores (the scale enters with the exponent)
+    auto cap_scores = [&](floatx4 (&sc)[QB][2]) {
+      const float cap = softcap / scale;
+#pragma unroll
+      for (int b = 0; b < QB; ++b)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) sc[b][h][i] = capped(sc[b][h][i], cap);
+    };
     // scores: S[key, query] = K Q^T, unscaled (the scale enters with the exponent)
     auto scores = [&](int stage, floatx4 (&sc)[QB][2]) {
       const unsigned char* kt = key_tiles + stage * KBYTES + key_fragment;
@@ -1287,6 +1299,7 @@ __global__ __launch_bounds__(MANY_WAVES ? 512 : 256, MANY_WAVES ? 1 : 2) void at
 #pragma unroll
           for (int b = 0; b < QB; ++b) sc[b][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kfrag, qf[b][c], sc[b][h], 0, 0, 0);
         }
+      if constexpr (CAPPED) cap_scores(sc);
     };
     // weights: as in attention_prefill_bf16_kernel; sc[b][h][i] belongs to key tile * 32 + 8 m + 4 h + i
     auto weights_with_maximum = [&](int tile, floatx4 (&sc)[QB][2], auto masked, bf16x8 (&pf)[QB]) {
@@ -1377,6 +1390,7 @@ __global__ __launch_bounds__(MANY_WAVES ? 512 : 256, MANY_WAVES ? 1 : 2) void at
       if (__any(again)) return false;
 #pragma unroll
       for (int b = 0; b < QB; ++b) run_sum[b] += tile_sum[b];
+      if constexpr (CAPPED) cap_scores(next);
       return true;
     };
     // values: O^T[dim, query] += V^T P
@@ -1573,7 +1587,6 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
   const DecodePrep prep{q_weight, nullptr, w_dtype == LRS_F32, eps, cosv, sinv, 0};
   LRS_REQUIRE(max_count >= 1 && max_count <= 32, "attention_prefill: query groups hold 1..32 tokens, got %d", max_count);
   LRS_REQUIRE(softcap >= 0.f, "attention_prefill: the cap on the scores must be positive (0 = none), got %g", (double)softcap);
-  LRS_REQUIRE(!(softcap > 0.f && prepare), "attention_prefill: capped scores come with prepared heads");
   LRS_REQUIRE(page_size % 16 == 0, "attention_prefill: page size %d is not a multiple of 16", page_size);
   LRS_REQUIRE(window >= 0 && keep_first >= 0 && (keep_first == 0 || (window > 0 && !prepare)),
               "attention_prefill: kept first positions (%d) need a window and prepared heads", keep_first);
@@ -1593,7 +1606,7 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
   const int span = window > 0 && window + 32 + 64 < max_context ? window + 32 + 64 : max_context;
   const size_t table_lds = sizeof(int) * (size_t)(span / page_size + 2);
   // (the kernel for heads of 128 reads the block table with scalar loads and keeps no copy)
-  LRS_REQUIRE((d == 128 && softcap == 0.f) || table_lds <= 24 * 1024, "attention_prefill: a context of %d tokens needs more block table entries than fit LDS", max_context);
+  LRS_REQUIRE(d == 128 || table_lds <= 24 * 1024, "attention_prefill: a context of %d tokens needs more block table entries than fit LDS", max_context);
   hipStream_t s = (hipStream_t)stream;
 #define LAUNCH2(D, QB)                                                                                               \
   attention_prefill_bf16_kernel<D, QB><<<grid, block, table_lds, s>>>((bf16*)out, out_stride, (const bf16*)q, q_stride, \
@@ -1609,10 +1622,6 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
     case 64: LAUNCH(64); break;
     case 96: LAUNCH(96); break;
     case 128:
-      if (softcap > 0.f) {       // capped scores: the kernel for any head size (the one below weaves the next tile's scores into this tile's weights)
-        LAUNCH(128);
-        break;
-      }
       // head size 128 has a kernel of its own, whose tiles go from memory straight into LDS
       // A kv group of five to eight heads: a wave for every head and one walk over the keys instead of two, while
       // the launch is small (measured, 40 heads on 8: 512 tokens 28.9 -> 19.6 us, 512 tokens after 1,536 88 -> 54 us;
@@ -1621,20 +1630,24 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
         const bool many = nq / nkv > 4 && (int64_t)n_blocks * nkv * splits <= 2 * compute_units();
         if (many) block = dim3((nq / nkv < 8 ? nq / nkv : 8) * WAVE);
 #define D128(QB, MANY, IDLE)                                                                                                      \
-        attention_prefill_d128_bf16_kernel<QB, MANY, IDLE><<<grid, block, 0, s>>>(                                                    \
+        if (softcap > 0.f) D128C(QB, MANY, IDLE, true);                                                                               \
+        else D128C(QB, MANY, IDLE, false)
+#define D128C(QB, MANY, IDLE, CAPPED)                                                                                             \
+        attention_prefill_d128_bf16_kernel<QB, MANY, IDLE, CAPPED><<<grid, block, 0, s>>>(                                            \
             (bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, \
             token_request, positions, qblock_token0, qblock_count, n_blocks, chunk, nq, nkv, page_size, scale, window, splits, slots, part_o, part_ml, \
-            prepare, prep, own_sinks)
-#define D128_OF(QB)                                      \
-        if (many && idle) D128(QB, true, true);          \
-        else if (many) D128(QB, true, false);            \
-        else if (idle) D128(QB, false, true);            \
-        else D128(QB, false, false)
+            prepare, prep, own_sinks, softcap)
+#define D128_OF(QB)                                        \
+        if (many && idle) { D128(QB, true, true); }        \
+        else if (many) { D128(QB, true, false); }          \
+        else if (idle) { D128(QB, false, true); }          \
+        else { D128(QB, false, false); }
         const bool idle = (nq / nkv) % (int)(block.x / WAVE) != 0;   // some wave of some pass has no head
         if (max_count <= 16) { D128_OF(1); }
         else { D128_OF(2); }
 #undef D128_OF
 #undef D128
+#undef D128C
       }
       break;
     case 192: LAUNCH(192); break;

@@ -1,6 +1,7 @@
 // Attention heads that are rotated first and normalised afterwards, and small kernels of layers built around them.
 //
-//   rotate_unit_prep   per token of the fused projection row [q: nq*d | k: nkv*d | v: nkv*dv | ...]: the first 2*rot_half dims
+//   rotate_unit_prep   per token of the fused projection row [q: nq*d | k: nkv*d | v: nkv*dv | ...]: a bias per column is added
+//                      (where the layer has one: the product before this kernel then leaves it out), the first 2*rot_half dims
 //                      of every q and k head are turned by the token's angles (pairs (j, j + rot_half), or neighbours
 //                      (2j, 2j + 1)), then the head is divided by its own root mean square over all d dims (no weight); q
 //                      written back in place, k into the key pages [page, kv_head, slot, d], v into the value pages
@@ -20,33 +21,34 @@ struct Item {
 };
 
 template <typename T>
-__device__ __forceinline__ Item rotated_item(const T* __restrict__ src, int j, int rot_half, int neighbours,
+__device__ __forceinline__ Item rotated_item(const T* __restrict__ src, const float* __restrict__ bias, int j, int rot_half, int neighbours,
                                              const float* __restrict__ cosrow, const float* __restrict__ sinrow) {
   Item it;
   if (j < rot_half) {
     it.first = neighbours ? 2 * j : j;
     it.second = neighbours ? 2 * j + 1 : j + rot_half;
-    const float u = to_float(src[it.first]), v = to_float(src[it.second]);
+    const float u = to_float(src[it.first]) + (bias ? bias[it.first] : 0.f), v = to_float(src[it.second]) + (bias ? bias[it.second] : 0.f);
     const float c = cosrow[j], s = sinrow[j];
     it.a = u * c - v * s;
     it.b = v * c + u * s;
   } else {
     it.first = j + rot_half;
     it.second = -1;
-    it.a = to_float(src[it.first]);
+    it.a = to_float(src[it.first]) + (bias ? bias[it.first] : 0.f);
     it.b = 0.f;
   }
   return it;
 }
 
-// A workgroup a token, a wave a head at a time.  The rotated values are made twice, once for the sum of squares and once
+// A workgroup four heads of a token, a wave a head (blockIdx.y counts the groups of four).  The rotated values are made twice, once for the sum of squares and once
 // for the write, by the same operations (the same bits); every value is read and written by one lane only, so q can be
 // written where it was read.
 template <typename T>
 __global__ __launch_bounds__(256) void rotate_unit_prep_kernel(T* __restrict__ qkv, int row_stride, int nq, int nkv, int d, int dv, float eps,
                                                                int unit, const float* __restrict__ cosv, const float* __restrict__ sinv,
                                                                int rot_half, int neighbours, T* __restrict__ k_pages,
-                                                               T* __restrict__ v_pages, const int* __restrict__ slots, int page_size) {
+                                                               T* __restrict__ v_pages, const int* __restrict__ slots, int page_size,
+                                                               const float* __restrict__ bias) {
   const int token = blockIdx.x, tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
   T* row = qkv + (int64_t)token * row_stride;
   const int slot = slots ? slots[token] : -1;
@@ -54,14 +56,15 @@ __global__ __launch_bounds__(256) void rotate_unit_prep_kernel(T* __restrict__ q
   const float* cosrow = cosv + (int64_t)token * rot_half;
   const float* sinrow = sinv + (int64_t)token * rot_half;
   const int items = d - rot_half;
-  for (int head = wave; head < nq + nkv; head += 4) {
+  const int head = blockIdx.y * 4 + wave;
+  if (head < nq + nkv) {
     const bool is_q = head < nq;
-    if (!is_q && slot < 0) continue;
     const T* src = row + (int64_t)head * d;
+    const float* hb = bias ? bias + (int64_t)head * d : nullptr;
     float ss = 0.f;
-    if (unit) {
+    if (unit && (is_q || slot >= 0)) {
       for (int j = lane; j < items; j += WAVE) {
-        const Item it = rotated_item(src, j, rot_half, neighbours, cosrow, sinrow);
+        const Item it = rotated_item(src, hb, j, rot_half, neighbours, cosrow, sinrow);
         ss = fmaf(it.a, it.a, ss);
         ss = fmaf(it.b, it.b, ss);
       }
@@ -69,17 +72,20 @@ __global__ __launch_bounds__(256) void rotate_unit_prep_kernel(T* __restrict__ q
     }
     const float inv = unit ? 1.0f / sqrtf(ss / (float)d + eps) : 1.f;
     T* dst = is_q ? row + (int64_t)head * d : k_pages + ((page * nkv + (head - nq)) * page_size + off) * d;
-    for (int j = lane; j < items; j += WAVE) {
-      const Item it = rotated_item(src, j, rot_half, neighbours, cosrow, sinrow);
-      dst[it.first] = from_float<T>(it.a * inv);
-      if (it.second >= 0) dst[it.second] = from_float<T>(it.b * inv);
+    if (is_q || slot >= 0) {
+      for (int j = lane; j < items; j += WAVE) {
+        const Item it = rotated_item(src, hb, j, rot_half, neighbours, cosrow, sinrow);
+        dst[it.first] = from_float<T>(it.a * inv);
+        if (it.second >= 0) dst[it.second] = from_float<T>(it.b * inv);
+      }
     }
   }
-  if (slot >= 0) {
+  if (slot >= 0) {           // the values, dealt out over the token's workgroups
     const int qn = nq * d, kn = nkv * d, vn = nkv * dv;
-    for (int e = tid; e < vn; e += 256) {
+    for (int e = blockIdx.y * 256 + tid; e < vn; e += 256 * gridDim.y) {
       const int kvh = e / dv, i = e % dv;
-      v_pages[((page * nkv + kvh) * dv + i) * page_size + off] = row[qn + kn + e];
+      const float v = to_float(row[qn + kn + e]) + (bias ? bias[qn + kn + e] : 0.f);
+      v_pages[((page * nkv + kvh) * dv + i) * page_size + off] = from_float<T>(v);
     }
   }
 }
@@ -93,7 +99,7 @@ __global__ __launch_bounds__(256) void rotate_unit_prep_vec_kernel(bf16* __restr
                                                                    float eps, int unit, const float* __restrict__ cosv,
                                                                    const float* __restrict__ sinv, int rot_half, int neighbours,
                                                                    bf16* __restrict__ k_pages, bf16* __restrict__ v_pages,
-                                                                   const int* __restrict__ slots, int page_size) {
+                                                                   const int* __restrict__ slots, int page_size, const float* __restrict__ bias) {
   const int token = blockIdx.x, tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
   bf16* row = qkv + (int64_t)token * row_stride;
   const int slot = slots ? slots[token] : -1;
@@ -104,10 +110,19 @@ __global__ __launch_bounds__(256) void rotate_unit_prep_vec_kernel(bf16* __restr
   // behind the rotated part; with neighbours, item j < rot_half / 4 is the run 8j (four pairs), the rest single runs
   const int paired = neighbours ? rot_half / 4 : rot_half / 8;
   const int items = neighbours ? d / 8 : (d - rot_half) / 8;
-  for (int head = wave; head < nq + nkv; head += 4) {
+  const int head = blockIdx.y * 4 + wave;
+  // eight values of a run with their biases added
+  auto run_of = [&](const bf16* at, const float* b, float (&out)[8]) {
+    const bf16x8 x = *(const bf16x8*)at;
+    floatx4 b0 = {0.f, 0.f, 0.f, 0.f}, b1 = b0;
+    if (b) b0 = *(const floatx4*)b, b1 = *(const floatx4*)(b + 4);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out[i] = (float)x[i] + (i < 4 ? b0[i] : b1[i - 4]);
+  };
+  if (head < nq + nkv && (head < nq || slot >= 0)) {
     const bool is_q = head < nq;
-    if (!is_q && slot < 0) continue;
     const bf16* src = row + (int64_t)head * d;
+    const float* hb = bias ? bias + (int64_t)head * d : nullptr;
     float va[RUNS][8], vb[RUNS][8];
     float ss = 0.f;
 #pragma unroll
@@ -115,7 +130,9 @@ __global__ __launch_bounds__(256) void rotate_unit_prep_vec_kernel(bf16* __restr
       const int j = lane + n * WAVE;
       if (j >= items) continue;
       if (j < paired && !neighbours) {
-        const bf16x8 lo = *(const bf16x8*)(src + j * 8), hi = *(const bf16x8*)(src + j * 8 + rot_half);
+        float lo[8], hi[8];
+        run_of(src + j * 8, hb ? hb + j * 8 : nullptr, lo);
+        run_of(src + j * 8 + rot_half, hb ? hb + j * 8 + rot_half : nullptr, hi);
         floatx4 c4[2], s4[2];
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
@@ -124,18 +141,19 @@ __global__ __launch_bounds__(256) void rotate_unit_prep_vec_kernel(bf16* __restr
         }
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-          const float u = (float)lo[i], v = (float)hi[i], c = c4[i / 4][i % 4], s = s4[i / 4][i % 4];
+          const float u = lo[i], v = hi[i], c = c4[i / 4][i % 4], s = s4[i / 4][i % 4];
           va[n][i] = u * c - v * s;
           vb[n][i] = v * c + u * s;
           ss = fmaf(va[n][i], va[n][i], ss);
           ss = fmaf(vb[n][i], vb[n][i], ss);
         }
       } else if (j < paired) {
-        const bf16x8 x = *(const bf16x8*)(src + j * 8);
+        float x[8];
+        run_of(src + j * 8, hb ? hb + j * 8 : nullptr, x);
         const floatx4 c4 = *(const floatx4*)(cosrow + j * 4), s4 = *(const floatx4*)(sinrow + j * 4);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float u = (float)x[2 * i], v = (float)x[2 * i + 1];
+          const float u = x[2 * i], v = x[2 * i + 1];
           va[n][2 * i] = u * c4[i] - v * s4[i];
           va[n][2 * i + 1] = v * c4[i] + u * s4[i];
           ss = fmaf(va[n][2 * i], va[n][2 * i], ss);
@@ -143,12 +161,9 @@ __global__ __launch_bounds__(256) void rotate_unit_prep_vec_kernel(bf16* __restr
         }
       } else {
         const int at = neighbours ? j * 8 : j * 8 + rot_half;
-        const bf16x8 x = *(const bf16x8*)(src + at);
+        run_of(src + at, hb ? hb + at : nullptr, va[n]);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          va[n][i] = (float)x[i];
-          ss = fmaf(va[n][i], va[n][i], ss);
-        }
+        for (int i = 0; i < 8; ++i) ss = fmaf(va[n][i], va[n][i], ss);
       }
     }
     ss = wave_sum(ss);
@@ -172,11 +187,12 @@ __global__ __launch_bounds__(256) void rotate_unit_prep_vec_kernel(bf16* __restr
       }
     }
   }
-  if (slot >= 0) {
+  if (slot >= 0) {           // the values, dealt out over the token's workgroups
     const int qn = nq * d, kn = nkv * d, vn = nkv * dv;
-    for (int e = tid; e < vn; e += 256) {
+    for (int e = blockIdx.y * 256 + tid; e < vn; e += 256 * gridDim.y) {
       const int kvh = e / dv, i = e % dv;
-      v_pages[((page * nkv + kvh) * dv + i) * page_size + off] = row[qn + kn + e];
+      const float v = (float)row[qn + kn + e] + (bias ? bias[qn + kn + e] : 0.f);
+      v_pages[((page * nkv + kvh) * dv + i) * page_size + off] = (bf16)v;
     }
   }
 }
@@ -209,10 +225,10 @@ __global__ void scale_values_kernel(float* __restrict__ x, int64_t count, float 
 // qkv [tokens, row_stride] in dtype: q (nq*d) | k (nkv*d) | v (nkv*dv) | anything else.  cos, sin [tokens, rot_half] float32
 // (rot_half 0: no rotation).  neighbours: the pairs are dims (2j, 2j + 1) instead of (j, j + rot_half).  unit: every head is
 // divided by sqrt(mean of its squares + eps) after the rotation.  slots[t] = page * page_size + offset (negative: the token's
-// key and value are not stored).
+// key and value are not stored).  bias (float32 [nq*d + nkv*d + nkv*dv], or null): added to q, k and v as they are read.
 LRS_API int lrs_rotate_unit_prep(void* qkv, int dtype, int tokens, int row_stride, int nq, int nkv, int d, int dv, float eps, int unit,
                                  const float* cosv, const float* sinv, int rot_half, int neighbours, void* k_pages, void* v_pages,
-                                 const int* slots, int page_size, void* stream) {
+                                 const int* slots, int page_size, const float* bias, void* stream) {
   LRS_REQUIRE(tokens > 0 && nq > 0 && nkv > 0 && d > 0 && dv > 0, "rotate_unit_prep: bad sizes tokens=%d nq=%d nkv=%d d=%d dv=%d", tokens, nq, nkv, d, dv);
   LRS_REQUIRE(row_stride >= nq * d + nkv * d + nkv * dv, "rotate_unit_prep: rows of %d hold fewer than q, k and v", row_stride);
   LRS_REQUIRE(rot_half >= 0 && 2 * rot_half <= d, "rotate_unit_prep: rotary width %d exceeds head_dim %d", 2 * rot_half, d);
@@ -220,16 +236,17 @@ LRS_API int lrs_rotate_unit_prep(void* qkv, int dtype, int tokens, int row_strid
   LRS_REQUIRE(!unit || eps > 0.f, "rotate_unit_prep: eps must be positive");
   LRS_REQUIRE(k_pages && v_pages && slots && page_size > 0, "rotate_unit_prep: cache write needs pages, slots and a page size");
   hipStream_t s = (hipStream_t)stream;
+  const dim3 grid(tokens, (nq + nkv + 3) / 4);
   if (dtype == LRS_F32)
-    rotate_unit_prep_kernel<float><<<tokens, 256, 0, s>>>((float*)qkv, row_stride, nq, nkv, d, dv, eps, unit, cosv, sinv, rot_half, neighbours,
-                                                          (float*)k_pages, (float*)v_pages, slots, page_size);
+    rotate_unit_prep_kernel<float><<<grid, 256, 0, s>>>((float*)qkv, row_stride, nq, nkv, d, dv, eps, unit, cosv, sinv, rot_half, neighbours,
+                                                        (float*)k_pages, (float*)v_pages, slots, page_size, bias);
   else if (dtype == LRS_BF16 && d % 8 == 0 && d <= 8 * WAVE * RUNS && rot_half % (neighbours ? 4 : 8) == 0 && row_stride % 8 == 0 &&
-           ((uintptr_t)qkv | (uintptr_t)cosv | (uintptr_t)sinv | (uintptr_t)k_pages) % 16 == 0)
-    rotate_unit_prep_vec_kernel<<<tokens, 256, 0, s>>>((bf16*)qkv, row_stride, nq, nkv, d, dv, eps, unit, cosv, sinv, rot_half, neighbours,
-                                                       (bf16*)k_pages, (bf16*)v_pages, slots, page_size);
+           ((uintptr_t)qkv | (uintptr_t)cosv | (uintptr_t)sinv | (uintptr_t)k_pages | (uintptr_t)bias) % 16 == 0)
+    rotate_unit_prep_vec_kernel<<<grid, 256, 0, s>>>((bf16*)qkv, row_stride, nq, nkv, d, dv, eps, unit, cosv, sinv, rot_half, neighbours,
+                                                     (bf16*)k_pages, (bf16*)v_pages, slots, page_size, bias);
   else if (dtype == LRS_BF16)
-    rotate_unit_prep_kernel<bf16><<<tokens, 256, 0, s>>>((bf16*)qkv, row_stride, nq, nkv, d, dv, eps, unit, cosv, sinv, rot_half, neighbours,
-                                                         (bf16*)k_pages, (bf16*)v_pages, slots, page_size);
+    rotate_unit_prep_kernel<bf16><<<grid, 256, 0, s>>>((bf16*)qkv, row_stride, nq, nkv, d, dv, eps, unit, cosv, sinv, rot_half, neighbours,
+                                                       (bf16*)k_pages, (bf16*)v_pages, slots, page_size, bias);
   else return lrs_fail("rotate_unit_prep: unknown dtype %d", dtype);
   return lrs_check_launch("rotate_unit_prep");
 }

@@ -129,7 +129,7 @@ _SIGNATURES = {
                                   c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_sigmoid_gate": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "lrs_rotate_unit_prep": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p, c_int, c_int,
-                                     c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+                                     c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p]),
     "lrs_gated_clamped": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_void_p]),
     "lrs_add_gathered": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p]),
     "lrs_scale_values": (c_int, [c_void_p, c_int64, c_float, c_void_p]),
@@ -1032,10 +1032,11 @@ def sigmoid_gate(out: torch.Tensor, gate: torch.Tensor) -> None:
 
 
 def rotate_unit_prep(qkv: torch.Tensor, nq: int, nkv: int, d: int, dv: int, eps: float, unit: bool, cos, sin, neighbours: bool,
-                     k_pages: torch.Tensor, v_pages: torch.Tensor, slots: torch.Tensor, page_size: int) -> None:
+                     k_pages: torch.Tensor, v_pages: torch.Tensor, slots: torch.Tensor, page_size: int, bias: torch.Tensor | None = None) -> None:
     """The rows of `qkv` [T, >= nq*d + nkv*d + nkv*dv] (q | k | v | whatever follows): the first 2 * cos.shape[1] dims of every q
     and k head rotated (pairs (j, j + half), or with `neighbours` (2j, 2j + 1)), then, with `unit`, every head divided by
-    sqrt(mean of its squares + eps); q in place, k and v into the pages."""
+    sqrt(mean of its squares + eps); q in place, k and v into the pages.  bias (float32, at least nq*d + nkv*d + nkv*dv values): added
+    to q, k and v as they are read (the product that made the rows then left it out)."""
     tokens = qkv.shape[0]
     stride = _rows(qkv, "qkv")
     _need(qkv.shape[1] >= (nq + nkv) * d + nkv * dv, "rotate_unit_prep: the rows hold fewer than q, k and v")
@@ -1049,9 +1050,11 @@ def rotate_unit_prep(qkv: torch.Tensor, nq: int, nkv: int, d: int, dv: int, eps:
     _need(k_pages.is_contiguous() and v_pages.is_contiguous() and k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype,
           "rotate_unit_prep: pages must be contiguous and of the activation dtype")
     _need(slots.dtype == torch.int32 and slots.numel() >= tokens and slots.is_contiguous(), "rotate_unit_prep: slots must be int32 [T]")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() >= (nq + nkv) * d + nkv * dv),
+          "rotate_unit_prep: the bias must be float32 and hold a value for every column of q, k and v")
     _launch("lrs_rotate_unit_prep", _dev(qkv, "qkv"), dtype_code(qkv.dtype), tokens, stride, nq, nkv, d, dv, float(eps), int(unit),
             None if cos is None else cos.data_ptr(), None if sin is None else sin.data_ptr(), rot_half, int(neighbours), _dev(k_pages, "k_pages"),
-            _dev(v_pages, "v_pages"), _dev(slots, "slots"), page_size, _stream())
+            _dev(v_pages, "v_pages"), _dev(slots, "slots"), page_size, None if bias is None else _dev(bias, "bias"), _stream())
 
 
 def gated_clamped(out: torch.Tensor, gate_up: torch.Tensor, alpha: float, limit: float) -> None:

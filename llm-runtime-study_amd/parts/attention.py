@@ -99,6 +99,7 @@ class GQAAttention(Part):
                              "capped scores and an output gate come without shared or key-made values and per-head norms before the rotation")
         if self.neighbours and qk_norm:
             raise ValueError("neighbouring pairs are rotated by the kernel that normalises after the rotation or not at all")
+        self.b_late = None
         self.gate_width = 0 if not output_gate else num_heads if output_gate == "head" else num_heads * self.value_dim
         self.sinks = None
         self.w_qkv = self.b_qkv = self.w_o = self.q_norm = self.k_norm = None
@@ -136,6 +137,8 @@ class GQAAttention(Part):
                 biases.append(biases[0].new_zeros(pad))
         self.w_qkv = torch.cat(stacked, 0).to(dtype).contiguous()
         self.b_qkv = torch.cat(biases, 0).to(dtype).contiguous() if self.bias else None
+        # the kernel that rotates and then normalises the heads adds the biases itself, in float32, as it reads the rows
+        self.b_late = torch.cat(biases, 0).float().contiguous() if self.bias and (self.unit_after or self.neighbours) else None
         if self.has_sink:
             self.sinks = weights["sink"].float().contiguous()
         self.w_o = weights["o_proj.weight"].to(dtype).contiguous()
@@ -331,10 +334,10 @@ class GQAAttention(Part):
         t, d, dv, nq, nkv = rows_of(x), self.head_dim, self.value_dim, self.num_heads, self.num_kv_heads
         gate_at = (nq + nkv) * d + nkv * dv
         qkv = ctx.scratch("attn_qkvg", (t, self.w_qkv.shape[0]), ctx.dtype)
-        linear(ctx, qkv, x, self.w_qkv, self.b_qkv)
+        linear(ctx, qkv, x, self.w_qkv, None if self.b_late is not None else self.b_qkv)
         if self.unit_after or self.neighbours:
             ops.rotate_unit_prep(qkv, nq, nkv, d, dv, self.qk_norm_eps, self.unit_after, cos, sin, self.neighbours, cache.k_pages, cache.v_pages,
-                                 group.slots, group.page_size)
+                                 group.slots, group.page_size, bias=self.b_late)
         else:
             ops.qkv_norm_prep(qkv, nq, nkv, d, dv, self.q_norm, self.k_norm, self.qk_norm_eps, cos, sin, cache.k_pages, cache.v_pages,
                               group.slots, group.page_size)
