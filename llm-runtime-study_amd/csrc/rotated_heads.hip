@@ -80,7 +80,7 @@ __global__ __launch_bounds__(256) void rotate_unit_prep_kernel(T* __restrict__ q
       }
     }
   }
-  if (slot >= 0) {           // the values, dealt out over the token's workgroups
+  if (slot >= 0 && v_pages) {           // the values, dealt out over the token's workgroups (null: values_in_runs_kernel stores them)
     const int qn = nq * d, kn = nkv * d, vn = nkv * dv;
     for (int e = blockIdx.y * 256 + tid; e < vn; e += 256 * gridDim.y) {
       const int kvh = e / dv, i = e % dv;
@@ -93,7 +93,16 @@ __global__ __launch_bounds__(256) void rotate_unit_prep_kernel(T* __restrict__ q
 // The same for bfloat16 heads whose size and rotated part are multiples of eight (sixteen for neighbouring pairs): 16 bytes a
 // load, a lane holds runs of eight dims (a run and its partner run where the pairs lie rot_half apart; one run of four pairs
 // where they are neighbours), which stay in registers between the sum of squares and the write.  A head of up to 512 dims.
+// A head of few items shares its wave with others: `lanes` (a power of two, at least the head's items, 64 at most) lanes a head,
+// 64 / lanes heads a wave, and the sum of squares goes round those lanes only (a head of 128 dims is 12 or 16 items: four heads
+// a wave, where a wave a head left three lanes in four idle).
 constexpr int RUNS = 4;      // work items a lane holds: 64 lanes x 4 items x up to 16 dims
+
+__host__ __device__ inline int lanes_of_head(int items) {
+  int lanes = 1;
+  while (lanes < items && lanes < WAVE) lanes *= 2;
+  return lanes;
+}
 
 __global__ __launch_bounds__(256) void rotate_unit_prep_vec_kernel(bf16* __restrict__ qkv, int row_stride, int nq, int nkv, int d, int dv,
                                                                    float eps, int unit, const float* __restrict__ cosv,
@@ -110,7 +119,8 @@ __global__ __launch_bounds__(256) void rotate_unit_prep_vec_kernel(bf16* __restr
   // behind the rotated part; with neighbours, item j < rot_half / 4 is the run 8j (four pairs), the rest single runs
   const int paired = neighbours ? rot_half / 4 : rot_half / 8;
   const int items = neighbours ? d / 8 : (d - rot_half) / 8;
-  const int head = blockIdx.y * 4 + wave;
+  const int lanes = lanes_of_head(items), per_wave = WAVE / lanes, own = lane % lanes;
+  const int head = (blockIdx.y * 4 + wave) * per_wave + lane / lanes;
   // eight values of a run with their biases added
   auto run_of = [&](const bf16* at, const float* b, float (&out)[8]) {
     const bf16x8 x = *(const bf16x8*)at;
@@ -127,7 +137,7 @@ __global__ __launch_bounds__(256) void rotate_unit_prep_vec_kernel(bf16* __restr
     float ss = 0.f;
 #pragma unroll
     for (int n = 0; n < RUNS; ++n) {
-      const int j = lane + n * WAVE;
+      const int j = own + n * lanes;
       if (j >= items) continue;
       if (j < paired && !neighbours) {
         float lo[8], hi[8];
@@ -166,12 +176,12 @@ __global__ __launch_bounds__(256) void rotate_unit_prep_vec_kernel(bf16* __restr
         for (int i = 0; i < 8; ++i) ss = fmaf(va[n][i], va[n][i], ss);
       }
     }
-    ss = wave_sum(ss);
+    for (int step = lanes / 2; step > 0; step /= 2) ss += __shfl_xor(ss, step, WAVE);      // among the head's own lanes
     const float inv = unit ? 1.0f / sqrtf(ss / (float)d + eps) : 1.f;
     bf16* dst = is_q ? row + (int64_t)head * d : k_pages + ((page * nkv + (head - nq)) * page_size + off) * d;
 #pragma unroll
     for (int n = 0; n < RUNS; ++n) {
-      const int j = lane + n * WAVE;
+      const int j = own + n * lanes;
       if (j >= items) continue;
       bf16x8 first;
 #pragma unroll
@@ -187,12 +197,53 @@ __global__ __launch_bounds__(256) void rotate_unit_prep_vec_kernel(bf16* __restr
       }
     }
   }
-  if (slot >= 0) {           // the values, dealt out over the token's workgroups
+  if (slot >= 0 && v_pages) {           // the values, dealt out over the token's workgroups (null: values_in_runs_kernel stores them)
     const int qn = nq * d, kn = nkv * d, vn = nkv * dv;
     for (int e = blockIdx.y * 256 + tid; e < vn; e += 256 * gridDim.y) {
       const int kvh = e / dv, i = e % dv;
       const float v = (float)row[qn + kn + e] + (bias ? bias[qn + kn + e] : 0.f);
       v_pages[((page * nkv + kvh) * dv + i) * page_size + off] = (bf16)v;
+    }
+  }
+}
+
+// The values of 16 consecutive tokens of the step and one kv head into the value pages [page, kv_head, dv, slot], for steps of
+// many tokens: tokens that follow each other inside a page lie side by side there, so a thread gathers one dim of 16 / sizeof(T)
+// such tokens (neighbouring lanes read neighbouring dims of one token), adds the dim's bias and writes one 16-byte store; where
+// a run is broken (a page's edge, another request, a slot that is not stored) it stores one by one.
+template <typename T>
+__global__ __launch_bounds__(256) void values_in_runs_kernel(const T* __restrict__ qkv, int row_stride, int v_offset, int tokens, int nkv, int dv,
+                                                             T* __restrict__ v_pages, const int* __restrict__ slots, int page_size,
+                                                             const float* __restrict__ bias) {
+  constexpr int RUN = 16 / sizeof(T);
+  typedef T vec __attribute__((ext_vector_type(RUN)));
+  __shared__ int slot_of[16];
+  const int tid = threadIdx.x, token0 = blockIdx.x * 16, kvh = blockIdx.y;
+  if (tid < 16) slot_of[tid] = token0 + tid < tokens ? slots[token0 + tid] : -1;
+  __syncthreads();
+  for (int e = tid; e < dv * (16 / RUN); e += 256) {
+    const int dim = e % dv, first = (e / dv) * RUN;
+    const int slot0 = slot_of[first];
+    bool run = slot0 >= 0 && slot0 % RUN == 0 && slot0 % page_size + RUN <= page_size;
+#pragma unroll
+    for (int i = 1; i < RUN; ++i) run = run && slot_of[first + i] == slot0 + i;
+    const int column = v_offset + kvh * dv + dim;
+    const float b = bias ? bias[column] : 0.f;
+    const T* src = qkv + (int64_t)(token0 + first) * row_stride + column;
+    if (run) {
+      vec v;
+#pragma unroll
+      for (int i = 0; i < RUN; ++i) v[i] = from_float<T>(to_float(src[(int64_t)i * row_stride]) + b);
+      const int64_t page = slot0 / page_size, off = slot0 % page_size;
+      *(vec*)(v_pages + ((page * nkv + kvh) * dv + dim) * page_size + off) = v;
+    } else {
+#pragma unroll
+      for (int i = 0; i < RUN; ++i) {
+        const int slot = slot_of[first + i];
+        if (slot < 0) continue;
+        const int64_t page = slot / page_size, off = slot % page_size;
+        v_pages[((page * nkv + kvh) * dv + dim) * page_size + off] = from_float<T>(to_float(src[(int64_t)i * row_stride]) + b);
+      }
     }
   }
 }
@@ -236,15 +287,29 @@ LRS_API int lrs_rotate_unit_prep(void* qkv, int dtype, int tokens, int row_strid
   LRS_REQUIRE(!unit || eps > 0.f, "rotate_unit_prep: eps must be positive");
   LRS_REQUIRE(k_pages && v_pages && slots && page_size > 0, "rotate_unit_prep: cache write needs pages, slots and a page size");
   hipStream_t s = (hipStream_t)stream;
-  const dim3 grid(tokens, (nq + nkv + 3) / 4);
+  dim3 grid(tokens, (nq + nkv + 3) / 4);
+  // steps of many tokens: the values as runs of slots, 16 bytes a store, by workgroups of their own (token by token they are
+  // 2-byte writes a page row apart)
+  if (tokens >= 64 && page_size % (dtype == LRS_F32 ? 4 : 8) == 0 && (uintptr_t)v_pages % 16 == 0) {
+    const dim3 vgrid((tokens + 15) / 16, nkv);
+    if (dtype == LRS_F32)
+      values_in_runs_kernel<float><<<vgrid, 256, 0, s>>>((const float*)qkv, row_stride, (nq + nkv) * d, tokens, nkv, dv, (float*)v_pages, slots, page_size, bias);
+    else if (dtype == LRS_BF16)
+      values_in_runs_kernel<bf16><<<vgrid, 256, 0, s>>>((const bf16*)qkv, row_stride, (nq + nkv) * d, tokens, nkv, dv, (bf16*)v_pages, slots, page_size, bias);
+    else return lrs_fail("rotate_unit_prep: unknown dtype %d", dtype);
+    if (lrs_check_launch("values_in_runs")) return 1;
+    v_pages = nullptr;
+  }
   if (dtype == LRS_F32)
     rotate_unit_prep_kernel<float><<<grid, 256, 0, s>>>((float*)qkv, row_stride, nq, nkv, d, dv, eps, unit, cosv, sinv, rot_half, neighbours,
                                                         (float*)k_pages, (float*)v_pages, slots, page_size, bias);
   else if (dtype == LRS_BF16 && d % 8 == 0 && d <= 8 * WAVE * RUNS && rot_half % (neighbours ? 4 : 8) == 0 && row_stride % 8 == 0 &&
-           ((uintptr_t)qkv | (uintptr_t)cosv | (uintptr_t)sinv | (uintptr_t)k_pages | (uintptr_t)bias) % 16 == 0)
+           ((uintptr_t)qkv | (uintptr_t)cosv | (uintptr_t)sinv | (uintptr_t)k_pages | (uintptr_t)bias) % 16 == 0) {
+    const int per_block = 4 * (WAVE / lanes_of_head(neighbours ? d / 8 : (d - rot_half) / 8));       // heads a workgroup takes
+    grid.y = (nq + nkv + per_block - 1) / per_block;
     rotate_unit_prep_vec_kernel<<<grid, 256, 0, s>>>((bf16*)qkv, row_stride, nq, nkv, d, dv, eps, unit, cosv, sinv, rot_half, neighbours,
                                                      (bf16*)k_pages, (bf16*)v_pages, slots, page_size, bias);
-  else if (dtype == LRS_BF16)
+  } else if (dtype == LRS_BF16)
     rotate_unit_prep_kernel<bf16><<<grid, 256, 0, s>>>((bf16*)qkv, row_stride, nq, nkv, d, dv, eps, unit, cosv, sinv, rot_half, neighbours,
                                                        (bf16*)k_pages, (bf16*)v_pages, slots, page_size, bias);
   else return lrs_fail("rotate_unit_prep: unknown dtype %d", dtype);
