@@ -42,6 +42,13 @@ __device__ __forceinline__ float with_sink(float sink2, float top, float& total)
 }
 constexpr float LOG2E = 1.4426950408889634f;
 
+// A gate a head: the head's output times sigmoid(gates[token, head]), the gate values lying in rows of their own stride (the
+// columns of the projection that made them).  Null: no gate.
+template <typename T>
+__device__ __forceinline__ float head_gate(const T* __restrict__ gates, int gate_stride, int64_t token, int head) {
+  return gates ? 1.0f / (1.0f + __expf(-(float)gates[token * gate_stride + head])) : 1.f;
+}
+
 // ---------------------------------------------------------- generic kernel
 // One workgroup per (query token, query head); any head_dim, values of any size dv up to 4 * threads.  keep_first: with a
 // window, the keys at positions below keep_first stay visible however far back they lie (they keep their positions).
@@ -51,7 +58,7 @@ __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
     const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_request,
     const int* __restrict__ positions, int nq, int nkv, int d, int dv, int page_size, float scale,
-    int window, int keep_first, const float* __restrict__ sinks, float softcap) {
+    int window, int keep_first, const float* __restrict__ sinks, float softcap, const T* __restrict__ gates, int gate_stride) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   float* qs = smem;                           // [d]
   float* probs = qs + d + d % 2;              // [THREADS]
@@ -148,7 +155,7 @@ __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
     keep = expf(running_max - top);
     running_sum = running_sum * keep + expf(sink - top);
   }
-  const float inv = keep / running_sum;
+  const float inv = keep / running_sum * head_gate(gates, gate_stride, token, head);
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
     const int dim = tid + c * THREADS;
@@ -263,7 +270,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_bf16_kernel(
     bf16* __restrict__ v_pages, const int* __restrict__ block_table, int table_stride,
     const int* __restrict__ token_request, const int* __restrict__ positions, int nq, int nkv,
     int page_size, float scale, int window, int splits, int slots, DecodePrep prep, const float* __restrict__ sinks,
-    float softcap) {
+    float softcap, const bf16* __restrict__ gates, int gate_stride) {
   constexpr int DS = D / 32, DB = D / 16, THREADS = WAVES * 64;
   __shared__ float sm_m[WAVES][16], sm_l[WAVES][16];
   __shared__ float sm_o[WAVES][D][16];
@@ -505,7 +512,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_bf16_kernel(
     const int head = kvh * group + h;
     if (slots <= 1) {
       if (sinks) acc *= with_sink(sinks[head] * LOG2E, top, total);
-      out[(int64_t)token * out_stride + (int64_t)head * D + dim] = (bf16)(acc / total);
+      out[(int64_t)token * out_stride + (int64_t)head * D + dim] = (bf16)(acc / total * head_gate(gates, gate_stride, token, head));
     } else {
       const int64_t slot = ((int64_t)token * nq + head) * slots + split;
       part_o[slot * D + dim] = acc;
@@ -523,7 +530,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_bf16_kernel(
 // write back and invalidate whole caches; measured, they cost many times what this kernel does.
 __global__ void attention_merge_kernel(bf16* __restrict__ out, int out_stride, const float* __restrict__ part_o,
                                        const float* __restrict__ part_ml, int nq, int d, int splits,
-                                       const float* __restrict__ sinks) {
+                                       const float* __restrict__ sinks, const bf16* __restrict__ gates, int gate_stride) {
   const int token = blockIdx.x, head = blockIdx.y;
   const int64_t base = ((int64_t)token * nq + head) * splits;
   // Everything is asked for before anything is used: the partial sums of a split do not wait for its maximum
@@ -556,7 +563,7 @@ __global__ void attention_merge_kernel(bf16* __restrict__ out, int out_stride, c
       }
     }
     if (sinks) acc *= with_sink(sinks[head] * LOG2E, top, total);
-    out[(int64_t)token * out_stride + (int64_t)head * d + dim] = (bf16)(acc / total);
+    out[(int64_t)token * out_stride + (int64_t)head * d + dim] = (bf16)(acc / total * head_gate(gates, gate_stride, token, head));
   }
 }
 
@@ -567,7 +574,7 @@ __global__ void attention_merge_kernel(bf16* __restrict__ out, int out_stride, c
 template <int SPLITS>
 __global__ __launch_bounds__(256) void attention_merge_wide_kernel(bf16* __restrict__ out, int out_stride, const float* __restrict__ part_o,
                                                                    const float* __restrict__ part_ml, int64_t quads, int nq, int d,
-                                                                   const float* __restrict__ sinks) {
+                                                                   const float* __restrict__ sinks, const bf16* __restrict__ gates, int gate_stride) {
   const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (e >= quads) return;
   const int per_head = d / 4;
@@ -602,26 +609,27 @@ __global__ __launch_bounds__(256) void attention_merge_wide_kernel(bf16* __restr
     for (int i = 0; i < 4; ++i) acc[i] *= keep;
   }
   bf16x4 r;
+  const float gate = head_gate(gates, gate_stride, token, (int)head);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) r[i] = (bf16)(acc[i] / total);
+  for (int i = 0; i < 4; ++i) r[i] = (bf16)(acc[i] / total * gate);
   *(bf16x4*)(out + token * out_stride + head * d + dim) = r;
 }
 
 static void launch_attention_merge(bf16* out, int out_stride, const float* part_o, const float* part_ml, int tokens, int nq, int d,
-                                   int splits, const float* sinks, hipStream_t s) {
+                                   int splits, const float* sinks, const bf16* gates, int gate_stride, hipStream_t s) {
   const bool wide = tokens >= 64 && d % 4 == 0 && out_stride % 4 == 0 && (uintptr_t)out % 8 == 0 && (uintptr_t)part_o % 16 == 0 &&
                     (uintptr_t)part_ml % 8 == 0 && (splits == 2 || splits == 3 || splits == 4 || splits == 5 || splits == 8 || splits == 9);
   if (wide) {
     const int64_t quads = (int64_t)tokens * nq * (d / 4);
     const int blocks = (int)((quads + 255) / 256);
-    if (splits == 2) attention_merge_wide_kernel<2><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d, sinks);
-    else if (splits == 3) attention_merge_wide_kernel<3><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d, sinks);
-    else if (splits == 4) attention_merge_wide_kernel<4><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d, sinks);
-    else if (splits == 5) attention_merge_wide_kernel<5><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d, sinks);
-    else if (splits == 9) attention_merge_wide_kernel<9><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d, sinks);
-    else attention_merge_wide_kernel<8><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d, sinks);
+    if (splits == 2) attention_merge_wide_kernel<2><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d, sinks, gates, gate_stride);
+    else if (splits == 3) attention_merge_wide_kernel<3><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d, sinks, gates, gate_stride);
+    else if (splits == 4) attention_merge_wide_kernel<4><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d, sinks, gates, gate_stride);
+    else if (splits == 5) attention_merge_wide_kernel<5><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d, sinks, gates, gate_stride);
+    else if (splits == 9) attention_merge_wide_kernel<9><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d, sinks, gates, gate_stride);
+    else attention_merge_wide_kernel<8><<<blocks, 256, 0, s>>>(out, out_stride, part_o, part_ml, quads, nq, d, sinks, gates, gate_stride);
   } else {
-    attention_merge_kernel<<<dim3(tokens, nq), d < 64 ? 64 : d, 0, s>>>(out, out_stride, part_o, part_ml, nq, d, splits, sinks);
+    attention_merge_kernel<<<dim3(tokens, nq), d < 64 ? 64 : d, 0, s>>>(out, out_stride, part_o, part_ml, nq, d, splits, sinks, gates, gate_stride);
   }
 }
 
@@ -709,7 +717,7 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
                                  int page_size, float scale, int window, int keep_first, int splits, int form, int prepare,
                                  const void* q_weight, const void* k_weight, int w_dtype, float eps,
                                  const float* cosv, const float* sinv, int kv_columns, const float* sinks, float softcap,
-                                 void* stream) {
+                                 const void* gates, int gate_stride, void* stream) {
   LRS_REQUIRE(tokens > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_decode: bad sizes tokens=%d nq=%d nkv=%d", tokens, nq, nkv);
   LRS_REQUIRE(nq / nkv <= 16, "attention_decode: %d query heads per kv head, at most 16 fit a tile", nq / nkv);
   LRS_REQUIRE(page_size % 16 == 0, "attention_decode: page size %d is not a multiple of 16", page_size);
@@ -742,7 +750,8 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
   // tile on the way while it works (heads of 192 dims have no registers for that and stay with 0)
 #define ARGS                                                                                                 \
   (bf16*)out, out_stride, part_o, part_ml, (const bf16*)q, q_stride, (bf16*)k_pages, (bf16*)v_pages, block_table, \
-      table_stride, token_request, positions, nq, nkv, page_size, scale, window, splits, slots, prep, slots == 1 ? sinks : nullptr, softcap
+      table_stride, token_request, positions, nq, nkv, page_size, scale, window, splits, slots, prep, slots == 1 ? sinks : nullptr, softcap, \
+      slots == 1 ? (const bf16*)gates : nullptr, gate_stride
 #define LAUNCH_PREP(D, PREP)                                                                                 \
   do {                                                                                                       \
     if (form == 2 && D <= 128) attention_decode_bf16_kernel<D, PREP, 8, (D <= 128)><<<grid, 512, table_lds, s>>>(ARGS); \
@@ -772,7 +781,7 @@ LRS_API int lrs_attention_decode(void* out, int out_stride, float* part_o, float
     if (lrs_check_launch("attention_kept")) return 1;
   }
   if (slots > 1) {
-    launch_attention_merge((bf16*)out, out_stride, part_o, part_ml, tokens, nq, d, slots, sinks, s);
+    launch_attention_merge((bf16*)out, out_stride, part_o, part_ml, tokens, nq, d, slots, sinks, (const bf16*)gates, gate_stride, s);
     return lrs_check_launch("attention_merge");
   }
   return 0;
@@ -806,7 +815,7 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
     const int* __restrict__ positions, const int* __restrict__ qblock_token0,
     const int* __restrict__ qblock_count, int n_blocks, int chunk, int nq, int nkv, int page_size, float scale,
     int window, int splits, int slots, float* __restrict__ part_o, float* __restrict__ part_ml,
-    const float* __restrict__ sinks, float softcap) {
+    const float* __restrict__ sinks, float softcap, const bf16* __restrict__ gates, int gate_stride) {
   constexpr int DS = D / 32, DB = D / 16;
   // Padded LDS rows.  Every fragment is read 16 bytes a lane, 16 rows at a time (the lane's row is col, its
   // piece g), which the LDS serves at its full 256 bytes a cycle when rows lie 32 bytes more than a multiple
@@ -1101,7 +1110,7 @@ __global__ __launch_bounds__(256, D <= 128 ? 2 : 1) void attention_prefill_bf16_
         }
       } else if (live[b]) {
         const float keep = sinks ? with_sink(sinks[head] * LOG2E, run_max[b] * scale2, total) : 1.f;
-        const float inv = keep / total;
+        const float inv = keep / total * head_gate(gates, gate_stride, token0 + b * 16 + col, head);
         bf16* dst = out + (int64_t)(token0 + b * 16 + col) * out_stride + (int64_t)head * D + g * 4;
 #pragma unroll
         for (int e = 0; e < DB; ++e) {
@@ -1144,7 +1153,7 @@ __global__ __launch_bounds__(MANY_WAVES ? 512 : 256, MANY_WAVES ? 1 : 2) void at
     const int* __restrict__ positions, const int* __restrict__ qblock_token0,
     const int* __restrict__ qblock_count, int n_blocks, int chunk, int nq, int nkv, int page_size, float scale,
     int window, int splits, int slots, float* __restrict__ part_o, float* __restrict__ part_ml, int prepare_q, DecodePrep prep,
-    const float* __restrict__ sinks, float softcap) {
+    const float* __restrict__ sinks, float softcap, const bf16* __restrict__ gates, int gate_stride) {
   constexpr int D = 128, DS = D / 32, DB = D / 16, STAGES = 3;
   constexpr int KBLOCK = 1024 + 32, KBYTES = 8 * KBLOCK, VHALF = 16 * D * 2 + 16, VBYTES = 2 * VHALF;
   constexpr int VSTAGE = (VBYTES + 63) / 64 * 64;
@@ -1517,7 +1526,7 @@ __global__ __launch_bounds__(MANY_WAVES ? 512 : 256, MANY_WAVES ? 1 : 2) void at
         }
       } else if (live[b]) {
         const float keep = sinks ? with_sink(sinks[head] * LOG2E, run_max[b] * scale2, total) : 1.f;
-        const float inv = keep / total;
+        const float inv = keep / total * head_gate(gates, gate_stride, token0 + b * 16 + col, head);
         bf16* dst = out + (int64_t)(token0 + b * 16 + col) * out_stride + (int64_t)head * D + g * 4;
 #pragma unroll
         for (int e = 0; e < DB; ++e) {
@@ -1575,7 +1584,8 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
                                   const int* qblock_count, int n_blocks, int max_count, int max_context, int nq,
                                   int nkv, int d, int page_size, float scale, int window, int keep_first, int tokens, int splits,
                                   float* part_o, float* part_ml, int prepare, const void* q_weight, int w_dtype, float eps,
-                                  const float* cosv, const float* sinv, const float* sinks, float softcap, void* stream) {
+                                  const float* cosv, const float* sinv, const float* sinks, float softcap, const void* gates,
+                                  int gate_stride, void* stream) {
   LRS_REQUIRE(n_blocks > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_prefill: bad sizes blocks=%d nq=%d nkv=%d", n_blocks, nq, nkv);
   if (prepare) {
     LRS_REQUIRE(lrs_attention_prefill_prepares(d), "attention_prefill: only the kernel for heads of 128 prepares the queries itself, got head_dim %d", d);
@@ -1592,6 +1602,7 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
               "attention_prefill: kept first positions (%d) need a window and prepared heads", keep_first);
   const int slots = splits + (keep_first > 0 ? 1 : 0);          // the kept keys' share is one more partial result
   const float* own_sinks = slots == 1 ? sinks : nullptr;          // with partial results the merge adds the sink
+  const bf16* own_gates = slots == 1 ? (const bf16*)gates : nullptr;   // ... and applies the gate
   LRS_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && out_stride % 4 == 0 && ((uintptr_t)out % 8) == 0,
               "attention_prefill: q rows must be 16-byte and out rows 8-byte aligned");
   // four waves (with fewer heads in a kv group the spare waves still help to bring tiles in), more only below
@@ -1613,7 +1624,7 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
                                                               (const bf16*)k_pages, (const bf16*)v_pages, block_table, \
                                                               table_stride, token_request, positions, qblock_token0, \
                                                               qblock_count, n_blocks, chunk, nq, nkv, page_size, scale, window, \
-                                                              splits, slots, part_o, part_ml, own_sinks, softcap)
+                                                              splits, slots, part_o, part_ml, own_sinks, softcap, own_gates, gate_stride)
 #define LAUNCH(D)                                \
   if (max_count <= 16) LAUNCH2(D, 1);            \
   else LAUNCH2(D, 2)
@@ -1636,7 +1647,7 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
         attention_prefill_d128_bf16_kernel<QB, MANY, IDLE, CAPPED><<<grid, block, 0, s>>>(                                            \
             (bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, \
             token_request, positions, qblock_token0, qblock_count, n_blocks, chunk, nq, nkv, page_size, scale, window, splits, slots, part_o, part_ml, \
-            prepare, prep, own_sinks, softcap)
+            prepare, prep, own_sinks, softcap, own_gates, gate_stride)
 #define D128_OF(QB)                                        \
         if (many && idle) { D128(QB, true, true); }        \
         else if (many) { D128(QB, true, false); }          \
@@ -1662,7 +1673,7 @@ LRS_API int lrs_attention_prefill(void* out, int out_stride, const void* q, int 
     if (lrs_check_launch("attention_kept")) return 1;
   }
   if (slots > 1) {
-    launch_attention_merge((bf16*)out, out_stride, part_o, part_ml, tokens, nq, d, slots, sinks, s);
+    launch_attention_merge((bf16*)out, out_stride, part_o, part_ml, tokens, nq, d, slots, sinks, (const bf16*)gates, gate_stride, s);
     return lrs_check_launch("attention_merge");
   }
   return 0;
@@ -1676,7 +1687,7 @@ LRS_API int lrs_attention(void* out, int out_stride, const void* q, int q_stride
                           const void* v_pages, const int* block_table, int table_stride,
                           const int* token_request, const int* positions, int dtype, int tokens,
                           int nq, int nkv, int d, int dv, int page_size, float scale, int window, int keep_first,
-                          const float* sinks, float softcap, void* stream) {
+                          const float* sinks, float softcap, const void* gates, int gate_stride, void* stream) {
   // value pages [P, nkv, dv, page]; out rows hold nq heads of dv values
   LRS_REQUIRE(tokens > 0 && nq > 0 && nkv > 0 && d > 0 && dv > 0 && page_size > 0, "attention: bad sizes tokens=%d nq=%d nkv=%d d=%d dv=%d page=%d", tokens, nq, nkv, d, dv, page_size);
   LRS_REQUIRE(nq % nkv == 0, "attention: %d query heads do not divide into %d kv heads", nq, nkv);
@@ -1690,11 +1701,11 @@ LRS_API int lrs_attention(void* out, int out_stride, const void* q, int q_stride
   if (dtype == LRS_F32)
     attention_generic_kernel<float, THREADS><<<grid, THREADS, lds, s>>>(
         (float*)out, out_stride, (const float*)q, q_stride, (const float*)k_pages, (const float*)v_pages,
-        block_table, table_stride, token_request, positions, nq, nkv, d, dv, page_size, scale, window, keep_first, sinks, softcap);
+        block_table, table_stride, token_request, positions, nq, nkv, d, dv, page_size, scale, window, keep_first, sinks, softcap, (const float*)gates, gate_stride);
   else if (dtype == LRS_BF16)
     attention_generic_kernel<bf16, THREADS><<<grid, THREADS, lds, s>>>(
         (bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)v_pages,
-        block_table, table_stride, token_request, positions, nq, nkv, d, dv, page_size, scale, window, keep_first, sinks, softcap);
+        block_table, table_stride, token_request, positions, nq, nkv, d, dv, page_size, scale, window, keep_first, sinks, softcap, (const bf16*)gates, gate_stride);
   else
     return lrs_fail("attention: unknown dtype %d", dtype);
   return lrs_check_launch("attention");

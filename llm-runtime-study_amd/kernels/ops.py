@@ -124,7 +124,7 @@ _SIGNATURES = {
                                             c_void_p, c_int64, c_void_p]),
     "lrs_norm_begin_parts": (c_int, [c_int]),
     "lrs_attention": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
-                              c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_float, c_void_p]),
+                              c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_float, c_void_p, c_int, c_void_p]),
     "lrs_qkv_norm_prep": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
                                   c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
     "lrs_sigmoid_gate": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
@@ -143,10 +143,10 @@ _SIGNATURES = {
                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "lrs_attention_decode": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                      c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int,
-                                     c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_void_p, c_float, c_void_p]),
+                                     c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_void_p, c_float, c_void_p, c_int, c_void_p]),
     "lrs_attention_prefill": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                                       c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
-                                      c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_float, c_void_p]),
+                                      c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int, c_void_p]),
     "lrs_attention_prefill_prepares": (c_int, [c_int]),
     "lrs_compute_units": (c_int, []),
     "lrs_gemm_lines_width": (c_int, [c_int, c_int, c_int]),
@@ -965,6 +965,14 @@ def scale_rows(out: torch.Tensor, x: torch.Tensor, sumsq: torch.Tensor, eps: flo
 
 
 # -------------------------------------------------------------- attention
+def _gates(gates: torch.Tensor | None, tokens: int, nq: int, dtype: torch.dtype, who: str) -> tuple:
+    """(address, row stride) of a gate a head, [T, nq] in the activation dtype, rows of any stride; (None, 0): no gate."""
+    if gates is None:
+        return None, 0
+    _need(gates.dim() == 2 and gates.shape == (tokens, nq) and gates.dtype == dtype and gates.stride(1) == 1, f"{who}: gates must be [{tokens}, {nq}] of the activation dtype")
+    return _dev(gates, "gates"), gates.stride(0)
+
+
 def _sinks(sinks: torch.Tensor | None, nq: int, who: str):
     if sinks is None:
         return None
@@ -974,11 +982,12 @@ def _sinks(sinks: torch.Tensor | None, nq: int, who: str):
 
 def attention(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
               token_request: torch.Tensor, positions: torch.Tensor, nq: int, scale: float, window: int = 0, keep_first: int = 0,
-              sinks: torch.Tensor | None = None, softcap: float = 0.0) -> None:
+              sinks: torch.Tensor | None = None, softcap: float = 0.0, gates: torch.Tensor | None = None) -> None:
     """out [T, nq*dv]; q [T, >= nq*d] (leading nq*d columns of each row); key pages [P, nkv, page, d],
     value pages [P, nkv, dv, page].  window: a token at p sees keys above p - window; keep_first: and those below keep_first.
     sinks (float32 [nq]): the softmax's denominator of head h has one more term exp(sinks[h]), without key or value.
-    softcap > 0: the scaled scores pass softcap * tanh(score / softcap) before the softmax."""
+    softcap > 0: the scaled scores pass softcap * tanh(score / softcap) before the softmax.
+    gates ([T, nq], rows of any stride): head h's output is multiplied by sigmoid(gates[t, h])."""
     tokens = out.shape[0]
     _need(k_pages.dim() == 4 and v_pages.dim() == 4 and k_pages.is_contiguous() and v_pages.is_contiguous(), "attention: pages must be contiguous")
     _, nkv, page_size, d = k_pages.shape
@@ -992,7 +1001,8 @@ def attention(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages
     _launch("lrs_attention", 
         _dev(out, "out"), _rows(out, "out"), _dev(q, "q"), _rows(q, "q"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"),
         _dev(block_table, "block_table"), block_table.stride(0), _dev(token_request, "token_request"), _dev(positions, "positions"),
-        dtype_code(q.dtype), tokens, nq, nkv, d, dv, page_size, scale, window, keep_first, _sinks(sinks, nq, "attention"), float(softcap), _stream())
+        dtype_code(q.dtype), tokens, nq, nkv, d, dv, page_size, scale, window, keep_first, _sinks(sinks, nq, "attention"), float(softcap),
+        *_gates(gates, tokens, nq, q.dtype, "attention"), _stream())
 
 
 def qkv_norm_prep(qkv: torch.Tensor, nq: int, nkv: int, d: int, dv: int, q_weight, k_weight, eps: float, cos, sin,
@@ -1139,7 +1149,7 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, 
                      token_request: torch.Tensor, positions: torch.Tensor, nq: int, scale: float, window: int = 0, splits: int = 1,
                      part_o: torch.Tensor | None = None, part_ml: torch.Tensor | None = None, max_context: int | None = None,
                      prepare: "DecodePrepare | None" = None, form: int = 0, keep_first: int = 0, sinks: torch.Tensor | None = None,
-                     softcap: float = 0.0) -> None:
+                     softcap: float = 0.0, gates: torch.Tensor | None = None) -> None:
     """attention() for a step with one query token per request, bfloat16 only; the keys of a token
     are divided between `splits` workgroups whose partial results meet in part_o / part_ml.
     keep_first (with a window and prepared heads): the first positions of a sequence stay visible behind the window; their
@@ -1182,7 +1192,7 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, 
         _dev(q, "q"), _rows(q, "q"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(block_table, "block_table"), block_table.stride(0),
         _dev(token_request, "token_request"), _dev(positions, "positions"), tokens,
         block_table.shape[1] * page_size if max_context is None else max_context, nq, nkv, d, page_size, scale, window, keep_first, splits,
-        form, *fused, _sinks(sinks, nq, "attention_decode"), float(softcap), _stream())
+        form, *fused, _sinks(sinks, nq, "attention_decode"), float(softcap), *_gates(gates, tokens, nq, q.dtype, "attention_decode"), _stream())
 
 
 def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
@@ -1190,7 +1200,7 @@ def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor,
                       nq: int, scale: float, window: int = 0, max_count: int | None = None, max_context: int | None = None,
                       splits: int = 1, part_o: torch.Tensor | None = None, part_ml: torch.Tensor | None = None,
                       prepare: "DecodePrepare | None" = None, keep_first: int = 0, sinks: torch.Tensor | None = None,
-                      softcap: float = 0.0) -> None:
+                      softcap: float = 0.0, gates: torch.Tensor | None = None) -> None:
     """attention() on matrix cores for any bfloat16 step.  qblock_token0 / qblock_count list groups of at
     most attention_prefill_group() consecutive tokens of one request that together cover every token of
     the step once; `max_count` is the largest count among them (the group limit if not given) and
@@ -1240,7 +1250,7 @@ def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_pages: torch.Tensor,
         attention_prefill_group() if max_count is None else max_count,
         block_table.shape[1] * page_size if max_context is None else max_context, nq, nkv, d, page_size, scale, window, keep_first,
         tokens, splits, None if slots == 1 else _dev(part_o, "part_o"), None if slots == 1 else _dev(part_ml, "part_ml"), *fused,
-        _sinks(sinks, nq, "attention_prefill"), float(softcap), _stream())
+        _sinks(sinks, nq, "attention_prefill"), float(softcap), *_gates(gates, tokens, nq, q.dtype, "attention_prefill"), _stream())
 
 
 def attention_prefill_prepares(d: int) -> bool:

@@ -27,7 +27,8 @@ And these, served by the same path: `unit_norm_after_rotation` divides every q a
 weight, `qk_norm_eps`) after the rotation instead of a weighted norm before it (`rotate_unit_prep` prepares the heads; the
 position part says whether a pair is (i, i + rot/2) or (2i, 2i + 1)); `sink` adds a learned term exp(sink_h) per head to the
 softmax's denominator, which has no key and no value; `score_cap` passes the scaled scores through cap * tanh(score / cap);
-`output_gate="head"` gates with one number a head, sigmoid(W_g x)_h, where `True` gates every value; `bias` with any of these
+`output_gate="head"` gates with one number a head, sigmoid(W_g x)_h, in the attention kernel that finishes a query or the merge
+of its partial results, where `True` gates every value by a kernel of its own; `bias` with any of these
 adds the stacked biases in the projection.
 """
 
@@ -342,6 +343,9 @@ class GQAAttention(Part):
             ops.qkv_norm_prep(qkv, nq, nkv, d, dv, self.q_norm, self.k_norm, self.qk_norm_eps, cos, sin, cache.k_pages, cache.v_pages,
                               group.slots, group.page_size)
         more = {"sinks": self.sinks, "softcap": self.score_cap or 0.0}
+        # a gate a head is applied by the attention kernel that finishes a query (or by the merge of its partial results); a
+        # gate a value by a kernel of its own behind them
+        gates = qkv[:, gate_at:gate_at + nq] if self.output_gate == "head" else None
         out = ctx.scratch("attn_out", (t, nq * dv), ctx.dtype)
         cores = dv == d and ops.attention_decode_supported(ctx.dtype, nq, nkv, d, group.page_size)
         extra = 1 if self.keep_first else 0      # the kept first positions' share is one more partial result for the merge
@@ -356,7 +360,7 @@ class GQAAttention(Part):
                 part_ml = ctx.scratch("attn_part_ml", (t, nq * (splits + extra) * 2), torch.float32)
             ops.attention_decode(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_slot, ctx.positions,
                                  nq, self.scale, self.window or 0, splits, part_o, part_ml, ctx.max_k_bound, None, form=1,
-                                 keep_first=self.keep_first, **more)
+                                 keep_first=self.keep_first, gates=gates, **more)
         elif cores:
             longest = ctx.max_k_bound if self.window is None else min(ctx.max_k_bound, self.window + 64)
             singles = ctx.single_rows
@@ -368,7 +372,7 @@ class GQAAttention(Part):
                     part_ml = ctx.scratch("attn_single_part_ml", (singles, nq * (splits + extra) * 2), torch.float32)
                 ops.attention_decode(out[:singles], qkv[:singles], cache.k_pages, cache.v_pages, group.block_table, ctx.token_slot,
                                      ctx.positions, nq, self.scale, self.window or 0, splits, part_o, part_ml, ctx.max_k_bound, None, form=1,
-                                     keep_first=self.keep_first, **more)
+                                     keep_first=self.keep_first, gates=None if gates is None else gates[:singles], **more)
             rest = ctx.memo.get("rows_after_singles")
             if rest is None:
                 rest = ctx.memo["rows_after_singles"] = (ctx.token_slot[singles:], ctx.positions[singles:])
@@ -379,11 +383,11 @@ class GQAAttention(Part):
                 part_ml = ctx.scratch("attn_part_ml", (t - singles, nq * (splits + extra) * 2), torch.float32)
             ops.attention_prefill(out[singles:], qkv[singles:], cache.k_pages, cache.v_pages, group.block_table, rest[0], rest[1],
                                   ctx.qblock_token0, ctx.qblock_count, nq, self.scale, self.window or 0, ctx.max_qblock, ctx.max_k_bound,
-                                  splits, part_o, part_ml, None, keep_first=self.keep_first, **more)
+                                  splits, part_o, part_ml, None, keep_first=self.keep_first, gates=None if gates is None else gates[singles:], **more)
         else:
             ops.attention(out, qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_slot, ctx.positions, nq, self.scale,
-                          self.window or 0, self.keep_first, **more)
-        if self.output_gate:
+                          self.window or 0, self.keep_first, gates=gates, **more)
+        if self.output_gate is True:
             ops.sigmoid_gate(out, qkv[:, gate_at:gate_at + self.gate_width])
         return linear(ctx, residual, out, self.w_o, accumulate=accumulate, then_norm=then_norm)
 
