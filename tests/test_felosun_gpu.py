@@ -448,6 +448,62 @@ def test_a_wider_model_through_the_products_for_many_rows(tmp_path, dtype):
     assert check(got, want, dtype) > 70
 
 
+def test_bfloat16_path_follows_float32_at_real_layer_sizes():
+    """Two layers at the sizes of a real model's (width 1,024, 16 heads of 128 on 8 key groups, a window of 512 with 8 kept
+    positions, 2 of 8 experts of 384 and a shared one, a vocabulary of 8,000): the bfloat16 path with everything it uses at that
+    size (graphs, the vendor's products for many rows, the grouped products' large tiles, key splits, the prefill kernel for
+    heads of 128 with capped scores, values stored as runs) against the float32 path of the same weights, over prompts in two
+    portions beside decoding requests and decode steps.  Experts are a discrete choice, so a share of the rows may differ."""
+    from llm_runtime_study_amd.benchmarks.shapes import SHAPES, felosun_like
+    from llm_runtime_study_amd.cache import CacheManager
+    from llm_runtime_study_amd.config import config_from_dict, spec_for
+    from llm_runtime_study_amd.engine.step import ModelRunner, StepEntry
+    from llm_runtime_study_amd.models import DecoderModel
+    from llm_runtime_study_amd.weights import random_init
+
+    raw = felosun_like(dict(SHAPES["0.6b"], vocab_size=8000), 2, experts=8, top=2, window=512, positions=2048)
+    cfg = config_from_dict(raw)
+    device = torch.device("cuda", 0)
+    weights = random_init.device_weights(DecoderModel(spec_for(cfg)), 0, torch.bfloat16, device, "scaled")
+    rng = np.random.default_rng(1)
+    prompts = [rng.integers(0, cfg.vocab_size, n).tolist() for n in (700, 33, 1500, 257, 64, 5, 1023, 90)]
+    tails = [rng.integers(0, cfg.vocab_size, 14).tolist() for _ in prompts]
+    logits_of = {}
+    for dtype in (torch.float32, torch.bfloat16):
+        model = DecoderModel(spec_for(cfg))
+        model.bind(weights, dtype)
+        cache = CacheManager(model.cache_needs(), page_size=16, num_pages=400, max_requests=8, max_seq_len=2048, dtype=dtype, device=device)
+        runner = ModelRunner(model, cache, max_step_tokens=2048, dtype=dtype, device=device, use_graph=dtype == torch.bfloat16)
+        rows = []
+        with torch.cuda.stream(torch.cuda.Stream(device)):
+            caches = [cache.admit(i) for i in range(len(prompts))]
+            fed = {}
+            for i, prompt in enumerate(prompts):
+                # the first half of the prompt beside one token of every earlier request, then the rest alone
+                half = len(prompt) // 2
+                decoding = [StepEntry(caches[j], [tails[j][fed[j]]], [0]) for j in sorted(fed)]
+                for j in fed:
+                    fed[j] += 1
+                mixed = runner.step(decoding + [StepEntry(caches[i], prompt[:half], [half - 1])])
+                rows.append(mixed.float().cpu())
+                rows.append(runner.step([StepEntry(caches[i], prompt[half:], [0, len(prompt) - half - 1])]).float().cpu())
+                fed[i] = 0
+            for _ in range(6):
+                rows.append(runner.step([StepEntry(caches[j], [tails[j][fed[j]]], [0]) for j in sorted(fed)]).float().cpu())
+                for j in fed:
+                    fed[j] += 1
+            if dtype == torch.bfloat16:
+                assert runner.graph_replays >= 3
+                runner.drop_graphs()
+        logits_of[dtype] = torch.cat(rows)
+        cache.check_invariants()
+        del runner, cache, model
+    exact, fast = logits_of[torch.float32], logits_of[torch.bfloat16]
+    assert exact.shape == fast.shape and exact.shape[0] > 80
+    error = (exact - fast).norm(dim=1) / exact.norm(dim=1)
+    assert (error < 3e-2).float().mean() >= 0.9 and error.median() < 1.5e-2, f"median {error.median():.3g}, {(error < 3e-2).float().mean():.2f} of the rows close"
+
+
 # ------------------------------------------------------------------------------------- planted inputs
 WINDOW, KEPT = 21, 3
 
