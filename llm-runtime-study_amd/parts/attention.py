@@ -29,7 +29,8 @@ position part says whether a pair is (i, i + rot/2) or (2i, 2i + 1)); `sink` add
 softmax's denominator, which has no key and no value; `score_cap` passes the scaled scores through cap * tanh(score / cap);
 `output_gate="head"` gates with one number a head, sigmoid(W_g x)_h, in the attention kernel that finishes a query or the merge
 of its partial results, where `True` gates every value by a kernel of its own; `bias` with any of these
-adds the stacked biases in the projection.
+adds the stacked biases to q, k and v: in the product's epilogue, or, where `rotate_unit_prep` prepares the heads, in that kernel
+as it reads the rows (in float32; the product then runs without a bias, through the vendor's library for many rows).
 """
 
 from __future__ import annotations
