@@ -80,10 +80,10 @@ class FelosunLayer:
     mlp: FelosunExperts | None
     rot_base: float | None = None
     rot_dims: int | None = None
-    rot_factor: float | None = None     # attention_2: every frequency divided by it
-    window: int | None = None           # attention
-    keep_first: int = 0                 # attention
-    softcap: float | None = None        # attention_2
+    rot_factor: float | None = None     # every frequency divided by it
+    window: int | None = None
+    keep_first: int = 0
+    softcap: float | None = None
     weights_of: int | None = None
 
     TYPES = ("attention", "attention_2")
@@ -111,24 +111,19 @@ class FelosunLayer:
             if made["rot_dims"] % 2 or made["rot_dims"] > made["dim"]:
                 raise ConfigError(f"{where}: rot.dims must be even and at most dim, got {made['rot_dims']}")
             if rot.get("scaling") is not None:
-                if kind != "attention_2":
-                    raise ConfigError(f"{where}: rot.scaling belongs to layers of type attention_2")
                 made["rot_factor"] = _positive_number(_section(rot, "scaling", where), "factor", where)
-        if kind == "attention":
-            if mixer.get("softcap") is not None:
-                raise ConfigError(f"{where}: softcap belongs to layers of type attention_2")
-            if mixer.get("mask") is not None:
-                mask = _section(mixer, "mask", where)
-                made["window"] = _positive(mask, "size", where)
-                kept = optional(mask, "keep_first", int, 0)
-                if kept < 0:
-                    raise ConfigError(f"{where}: mask.keep_first must not be negative, got {kept}")
-                made["keep_first"] = kept
-        else:
-            if mixer.get("mask") is not None:
-                raise ConfigError(f"{where}: a mask belongs to layers of type attention")
-            if mixer.get("softcap") is not None:
-                made["softcap"] = _positive_number(mixer, "softcap", where)
+        # The constants below are written for one type each in the design (the window for "attention", the cap and the stretched
+        # positions for "attention_2"); every mechanism is a parameter of the same mixer, so a file that gives one to the other
+        # type is served as it says.
+        if mixer.get("mask") is not None:
+            mask = _section(mixer, "mask", where)
+            made["window"] = _positive(mask, "size", where)
+            kept = optional(mask, "keep_first", int, 0)
+            if kept < 0:
+                raise ConfigError(f"{where}: mask.keep_first must not be negative, got {kept}")
+            made["keep_first"] = kept
+        if mixer.get("softcap") is not None:
+            made["softcap"] = _positive_number(mixer, "softcap", where)
         shared = raw.get("weights_of")
         if shared is not None and (not isinstance(shared, int) or isinstance(shared, bool)):
             raise ConfigError(f"{where}: weights_of must be a layer's number")

@@ -7,6 +7,7 @@ is grouped-query attention whose q and k heads are rotated first and then divide
                  positions visible; a learned sink per head in the softmax's denominator;
   "attention_2"  no biases; dims (i, i + rot/2) rotated with every frequency divided by a constant; the scaled scores capped
                  by cap * tanh(score / cap); the whole context; one sigmoid gate per head on the heads' outputs.
+(The window, the cap and the stretched positions are constants of a layer's entry: a layer of either kind has what its entry gives.)
 The feed-forward is a set of routed experts chosen by their largest sigmoid scores, each run on its score times the
 token (not weighted afterwards, not renormalised), with a clamped gated activation, and a shared expert beside them.  A layer
 may run with another layer's weights and a cache of its own: such a layer is a second schedule entry of the layer it names.
@@ -38,7 +39,7 @@ def _mixer(config: FelosunConfig, layer: FelosunLayer) -> PartSpec:
     first = layer.type == "attention"
     position = PartSpec("none")
     if layer.rot_dims is not None and first:
-        position = PartSpec("rope_interleaved", {"rotary_dim": layer.rot_dims, "theta": layer.rot_base})
+        position = PartSpec("rope_interleaved", {"rotary_dim": layer.rot_dims, "theta": layer.rot_base, "factor": layer.rot_factor or 1.0})
     elif layer.rot_dims is not None:
         position = PartSpec("rope_half", {"rotary_dim": layer.rot_dims, "theta": layer.rot_base, "factor": layer.rot_factor or 1.0})
     return PartSpec("gqa_attention", {

@@ -78,27 +78,30 @@ def yarn_frequencies(rotary_dim: int, theta: float, factor: float, original: flo
 class RotaryInterleaved(Part):
     """Rotary positions whose pairs are neighbours, (2i, 2i + 1): the pair (u, v) at position p becomes
     (u cos a - v sin a, v cos a + u sin a) with a = p * f_i, f_i = theta^(-2i / rotary_dim).  `scaling` (a mapping with
-    factor, original, fast, slow) stretches the slow pairs, see yarn_frequencies().  The tables are the same kind as the
+    factor, original, fast, slow) stretches the slow pairs, see yarn_frequencies(); `factor` alone divides every frequency by a
+    constant (linear scaling of the positions).  The tables are the same kind as the
     half-split part's, [T, rotary_dim / 2] float32 made once a step; the mixer's kernel pairs the dims."""
 
     pairing = "interleaved"
 
-    def __init__(self, rotary_dim: int, theta: float, scaling: dict | None = None):
+    def __init__(self, rotary_dim: int, theta: float, scaling: dict | None = None, factor: float = 1.0):
         if rotary_dim <= 0 or rotary_dim % 2 != 0:
             raise ValueError(f"rotary_dim must be a positive even integer, got {rotary_dim}")
         if theta <= 0 or theta == 1:
             raise ValueError(f"theta must be positive and not 1, got {theta}")
-        self.rotary_dim, self.theta = rotary_dim, theta
+        if not factor > 0 or (factor != 1.0 and scaling is not None):
+            raise ValueError(f"factor must be positive and comes without `scaling`, got {factor}")
+        self.rotary_dim, self.theta, self.factor = rotary_dim, theta, float(factor)
         self.scaling = None if scaling is None else tuple(float(scaling[name]) for name in ("factor", "original", "fast", "slow"))
         if self.scaling is None:
-            frequencies, self.magnitude = theta ** (-2.0 * torch.arange(0, rotary_dim // 2, dtype=torch.float64) / rotary_dim), 1.0
+            frequencies, self.magnitude = theta ** (-2.0 * torch.arange(0, rotary_dim // 2, dtype=torch.float64) / rotary_dim) / self.factor, 1.0
         else:
             frequencies, self.magnitude = yarn_frequencies(rotary_dim, theta, *self.scaling)
         self._inv_freq_host = frequencies.to(torch.float32)
         self._inv_freq = None
 
     def key(self):
-        return ("rope_interleaved", self.rotary_dim, self.theta, self.scaling)
+        return ("rope_interleaved", self.rotary_dim, self.theta, self.scaling, self.factor)
 
     def tables(self, ctx):
         """cos and sin [T, rotary_dim/2] float32 for this step's positions, times the magnitude (made once per step)."""
@@ -107,7 +110,7 @@ class RotaryInterleaved(Part):
             if self._inv_freq is None or self._inv_freq.device != ctx.positions.device:
                 self._inv_freq = self._inv_freq_host.to(ctx.positions.device)
             half = self.rotary_dim // 2
-            tag = f"{self.rotary_dim}_{self.theta}_{self.scaling}"
+            tag = f"{self.rotary_dim}_{self.theta}_{self.scaling}" + ("" if self.factor == 1.0 else f"_{self.factor}")
             cos = ctx.scratch(f"rope_pairs_cos_{tag}", (ctx.T, half), torch.float32)
             sin = ctx.scratch(f"rope_pairs_sin_{tag}", (ctx.T, half), torch.float32)
             ops.rope_table(cos, sin, ctx.positions, self._inv_freq, self.magnitude)

@@ -65,9 +65,10 @@ def visible(i: int, j: int, mask: dict | None) -> bool:
 
 
 def attention(x: torch.Tensor, w: dict, m: dict, eps: float, kind: str, weights_out: list | None = None) -> torch.Tensor:
-    """Both attention mixers.  kind "attention": biases, neighbouring pairs, window with kept first positions, a sink in the
-    denominator.  kind "attention_2": no biases, half-split pairs with linear scaling, a tanh cap on the scores, full causal
-    mask, a sigmoid gate per head.  In both, q and k are made unit-RMS per head after the rotation."""
+    """Both attention mixers.  kind "attention": biases, neighbouring pairs, a sink in the denominator (and, as a rule, a window
+    with kept first positions).  kind "attention_2": no biases, half-split pairs, a sigmoid gate per head (and, as a rule,
+    linear scaling, a tanh cap on the scores, the whole context).  In both, q and k are made unit-RMS per head after the
+    rotation, and the constants a layer's entry gives (mask, softcap, rot.scaling) are what it has."""
     n = x.shape[0]
     heads, groups, d, e = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     first = kind == "attention"
@@ -77,8 +78,7 @@ def attention(x: torch.Tensor, w: dict, m: dict, eps: float, kind: str, weights_
     q, k, v = q.view(n, heads, d), k.view(n, groups, d), v.view(n, groups, e)
     layout = "neighbours" if first else "halves"
     q, k = unit_rms(turn(q, m.get("rot"), layout), eps), unit_rms(turn(k, m.get("rot"), layout), eps)
-    mask = m.get("mask") if first else None
-    cap = None if first else m.get("softcap")
+    mask, cap = m.get("mask"), m.get("softcap")      # written for one kind each; a layer that is given the other's has it
     out = torch.zeros(n, heads, e, dtype=x.dtype)
     for h in range(heads):
         g = h // (heads // groups)

@@ -94,9 +94,9 @@ def test_refusals_name_the_layer():
     assert "heads" in refused(lambda raw: raw["layers"][0]["mixer"].update(heads=5))
     assert "rot.dims" in refused(lambda raw: raw["layers"][0]["mixer"]["rot"].update(dims=7))
     assert "rot.dims" in refused(lambda raw: raw["layers"][0]["mixer"]["rot"].update(dims=22))
-    assert "scaling" in refused(lambda raw: raw["layers"][1]["mixer"]["rot"].update(scaling={"factor": 2.0}))
-    assert "softcap" in refused(lambda raw: raw["layers"][1]["mixer"].update(softcap=5.0))
-    assert "mask" in refused(lambda raw: raw["layers"][0]["mixer"].update(mask={"size": 4}))
+    assert "factor" in refused(lambda raw: raw["layers"][0]["mixer"]["rot"].update(scaling={"factor": 0.0}))
+    assert "softcap" in refused(lambda raw: raw["layers"][0]["mixer"].update(softcap=-5.0))
+    assert "size" in refused(lambda raw: raw["layers"][1]["mixer"]["mask"].pop("size"))
     assert "top" in refused(lambda raw: raw["layers"][0]["mlp"]["router"].update(top=6))
     assert "limit" in refused(lambda raw: raw["layers"][0]["mlp"]["expert"].pop("limit"))
     assert "kind" in refused(lambda raw: raw["layers"][0]["mlp"].update(kind="dense"))
@@ -107,6 +107,24 @@ def test_refusals_name_the_layer():
     assert "must equal" in refused(lambda raw: raw["layers"][3]["mixer"].update(scale=0.5))
     assert "max_positions" in refused(lambda raw: raw.pop("max_positions"))
     assert "eps" in refused(lambda raw: raw["norm"].update(eps=0.0))
+
+
+def test_a_constant_given_to_the_other_type_is_served():
+    """The window is written for one type of layer, the cap and the stretched positions for the other; each is a parameter of
+    the same mixer, so a file that gives one to the other type gets it."""
+    from llm_runtime_study_amd.config import config_from_dict, spec_for
+
+    raw = copy.deepcopy(configs.ODD)
+    raw["layers"][1]["mixer"]["rot"]["scaling"] = {"factor": 2.0}
+    raw["layers"][1]["mixer"]["softcap"] = 5.0
+    raw["layers"][0]["mixer"]["mask"] = {"size": 4, "keep_first": 1}
+    raw["layers"][3], raw["layers"][4] = configs.shares(raw["layers"][0], 0), configs.shares(raw["layers"][1], 1)
+    config = config_from_dict(raw)
+    assert config.to_json_dict() == raw
+    spec = spec_for(config)
+    first, second = spec.layers[0].params["mixer"].params, spec.layers[1].params["mixer"].params
+    assert first["window"] == 4 and first["keep_first"] == 1 and first["score_cap"] == 4.0 and first["output_gate"] == "head"
+    assert second["score_cap"] == 5.0 and second["position"].params["factor"] == 2.0 and second["sink"] is True
 
 
 def test_context_length_is_bounded_by_the_learned_positions():

@@ -166,6 +166,35 @@ def test_capped_attention_with_head_gates_part(dtype, heads, groups, d, e, scale
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,groups,d,e", [(4, 2, 64, 64), (2, 1, 128, 128), (3, 1, 24, 40)])
+def test_every_constant_on_either_kind_part(dtype, heads, groups, d, e):
+    """A window with kept positions, a cap and stretched positions are parameters of one mixer: the kind with sinks and biases
+    under a cap and stretched positions, the kind with head gates behind a window with kept positions (the gate then meets the
+    kept positions' share in the merge of partial results)."""
+    from llm_runtime_study_amd.parts import PartSpec, create
+
+    width = 56
+    sizes = {"hidden_size": width, "num_heads": heads, "num_kv_heads": groups, "head_dim": d, "value_dim": e, "unit_norm_after_rotation": True,
+             "qk_norm_eps": 1e-4, "scale": 0.15, "window": 19, "keep_first": 4, "score_cap": 1.5}
+    m = {"heads": heads, "kv_heads": groups, "dim": d, "vdim": e, "scale": 0.15, "mask": {"size": 19, "keep_first": 4}, "softcap": 1.5,
+         "rot": {"base": 300.0, "dims": 8, "scaling": {"factor": 3.0}}}
+    inputs = {key: bf16_values(n, width, seed=500 + i) for i, (key, n) in enumerate(LENGTHS.items())}
+    for kind in ("attention", "attention_2"):
+        first = kind == "attention"
+        position = PartSpec("rope_interleaved" if first else "rope_half", {"rotary_dim": 8, "theta": 300.0, "factor": 3.0})
+        part = create("mixer", PartSpec("gqa_attention", dict(sizes, position=position, bias=first, sink=first, output_gate=False if first else "head")))
+        w = part_weights(part, 90)
+        if not first:
+            w["g_proj.weight"] = (w["g_proj.weight"] * 4.0).to(torch.bfloat16).double()
+        named = bound(part, w, dtype)
+        want = {key: plain.attention(x, named, m, 1e-4, kind) for key, x in inputs.items()}
+        for page_size in (16, 4):
+            got, _ = step_through(part, dtype, inputs, width, page_size=page_size)
+            for key in inputs:
+                close(got[key], want[key][:got[key].shape[0]], dtype, f32=5e-5, bf16=2e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("splits", ["few keys", "many keys"])
 def test_a_sink_that_outweighs_every_key_and_one_that_weighs_nothing(dtype, splits):
     """Heads of the matrix cores' shape: the first head's sink towers over every score (its output is nothing), the second's
