@@ -171,6 +171,10 @@ class FelosunConfig:
         if not isinstance(entries, list) or not entries:
             raise ConfigError("layers must be a non-empty list")
         eps = _positive_number(_section(raw, "norm", "config.json"), "eps", "config.json norm")
+        # what the entry of a layer that runs with another's weights leaves out (its feed-forward, say) is the owner's
+        entries = [dict(entries[layer["weights_of"]], **layer) if isinstance(layer, dict) and isinstance(layer.get("weights_of"), int)
+                   and not isinstance(layer.get("weights_of"), bool) and 0 <= layer["weights_of"] < len(entries)
+                   and isinstance(entries[layer["weights_of"]], dict) else layer for layer in entries]
         layers = tuple(FelosunLayer.from_dict(layer, index) for index, layer in enumerate(entries))
         for index, layer in enumerate(layers):
             if layer.weights_of is None:

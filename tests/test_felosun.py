@@ -76,6 +76,9 @@ def test_what_the_file_leaves_out_does_not_exist():
     first, second, third = config.layers[:3]
     assert first.softcap is None and first.rot_factor is None and first.mlp.shared_ff is None
     assert second.window is None and second.keep_first == 0 and third.rot_dims is None
+    # the entry of a layer that runs with another's weights may leave out what equals the owner's
+    del raw["layers"][4]["mlp"]
+    assert config_from_dict(raw).layers[4].mlp == config.layers[1].mlp
 
 
 def refused(change):
